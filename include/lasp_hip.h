@@ -1,0 +1,118 @@
+/*
+ * lasp_hip.h -- C ABI of liblasp_hip.so (gfx950 / MI355X).
+ *
+ * Causal decayed linear attention ("lightning attention") on one chunk of a
+ * sequence, forward and backward, with an optional d x e fp32 state arriving
+ * from the previous chunk (KV) and, in backward, from the next chunk (DKV).
+ *
+ * Tensor contract (all pointers are DEVICE pointers, all tensors contiguous,
+ * row-major):
+ *     q, k, dq, dk : (b, h, n, d)      element type `dtype`
+ *     v, o, do, dv : (b, h, n, e)      element type `dtype`
+ *     s            : h floats          per-head decay slope, >= 0
+ *     kv_in, kv_out, dkv_in, dkv_out : (b, h, d, e) float, may be NULL
+ *     seg states   : (b, h, n_seg, d, e) float workspace (see lasp_plan)
+ *
+ * Every call only ENQUEUES work on `stream` (a hipStream_t; NULL = the default
+ * stream); nothing is allocated, freed or synchronised, pointers are borrowed
+ * until the enqueued work has run.  Return value: 0 on success, > 0 a
+ * hipError_t, < 0 an argument error (LASP_E_*); lasp_last_error() then holds a
+ * message for the calling thread.
+ *
+ * The entry points replace the Triton launches of the reference:
+ *   lasp_chunk_fwd  <- lasp/lightning_attention.py:414-429 (_fwd_kernel, no state)
+ *                      lasp/lasp_fuse.py:380-399 (_fwd_kernel with KV in/out)
+ *                      lasp/lasp_fuse_parallel.py:852-942 (diag / kv_parallel /
+ *                        kv_reduce / none_diag launches + the torch KV update)
+ *   lasp_chunk_bwd  <- lasp/lightning_attention.py:459-502 (_bwd_intra_kernel,
+ *                        _bwd_inter_kernel)
+ *                      lasp/lasp_fuse.py:438-461 (_bwd_kernel with KV, DKV)
+ *                      lasp/lasp_fuse_parallel.py:970-1068
+ */
+#ifndef LASP_HIP_H
+#define LASP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LASP_ABI_VERSION 1
+
+/* element types of q/k/v/o/do/dq/dk/dv */
+#define LASP_DTYPE_F32 0
+#define LASP_DTYPE_BF16 1
+#define LASP_DTYPE_F16 2
+
+/* argument errors (negative return values) */
+#define LASP_E_NULL (-1)     /* a required pointer is NULL */
+#define LASP_E_SHAPE (-2)    /* unsupported b/h/n/d/e */
+#define LASP_E_DTYPE (-3)    /* unknown dtype code */
+#define LASP_E_SEGMENT (-4)  /* seg_len invalid for this shape */
+#define LASP_E_WORKSPACE (-5)/* workspace missing or too small */
+
+/* Which kernel family a shape/dtype is served by (lasp_kernel_path). */
+#define LASP_PATH_GENERIC 0 /* fp32-FMA kernels: any dtype, any n, d,e <= 128 */
+#define LASP_PATH_MFMA 1    /* bf16 MFMA kernels: bf16, d = e = 128, n % 64 == 0 */
+
+int lasp_abi_version(void);
+
+/* Message of the last failing call made by this thread ("" if none). */
+const char *lasp_last_error(void);
+
+/*
+ * Work decomposition.  A chunk of n tokens is cut into n_seg segments of
+ * seg_len tokens (the last one may be shorter); segments of one (b, h) run in
+ * parallel and are stitched by a decayed scan over their d x e states.
+ * lasp_plan returns the default seg_len for a shape (pass it, or any other
+ * positive multiple of 64, to the calls below); n_seg = ceil(n / seg_len) and
+ * the byte size of ONE segment-state array are written through the pointers
+ * (either may be NULL).  Replaces the BLOCK/NUM_BLOCK choice of
+ * lasp/lasp_fuse_parallel.py:1080-1085 and the `kv` buffer shape of :876.
+ */
+int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0,
+              int *seg_len, int *n_seg, size_t *state_bytes);
+
+/* LASP_PATH_* for this shape, or a negative LASP_E_* if it is unsupported. */
+int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype);
+
+/*
+ * Forward:  O = ((Q K^T) (.) M) V + diag(l^i) Q KV_in,   M_ij = l^(i-j) [j <= i]
+ *           KV_out = l^n KV_in + sum_j l^(n-j) k_j^T v_j              (l = exp(-s_h))
+ * kv_in  NULL = zero incoming state.  kv_out NULL = state not wanted.
+ * kv_out may alias kv_in (in-place update, as lasp/lasp_fuse.py:126-127).
+ * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds the
+ * state entering each segment (segment 0: KV_in), which lasp_chunk_bwd accepts
+ * as `kv_seg_states` to skip recomputing it.  It may be NULL only when
+ * n_seg == 1 and kv_in == NULL and kv_out == NULL.
+ */
+int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s,
+                   const float *kv_in, float *kv_out, void *o, float *seg_states,
+                   int b, int h, int64_t n, int d, int e, int dtype, int seg_len,
+                   void *stream);
+
+/*
+ * Backward (given dO and DKV_in = dL/dKV_out):
+ *   dQ_i = sum_{j<=i} l^(i-j) (dO_i . v_j) k_j + l^i dO_i KV_in^T
+ *   dK_j = sum_{i>=j} l^(i-j) (dO_i . v_j) q_i + l^(n-j) v_j DKV_in^T
+ *   dV_j = sum_{i>=j} l^(i-j) (q_i . k_j) dO_i + l^(n-j) k_j DKV_in
+ *   DKV_out = l^n DKV_in + sum_i l^i q_i^T dO_i                  (= dL/dKV_in)
+ * kv_in / dkv_in NULL = zero.  dkv_out NULL = not wanted; may alias dkv_in
+ * (lasp/lasp_fuse.py:352-353).
+ * kv_seg_states: the array lasp_chunk_fwd left in `seg_states` for the same
+ * inputs, seg_len and kv_in, or NULL to recompute it (then `workspace` must
+ * hold 2 * state_bytes, else 1 * state_bytes).
+ */
+int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
+                   const void *d_o, const float *kv_in, const float *dkv_in,
+                   void *dq, void *dk, void *dv, float *dkv_out,
+                   const float *kv_seg_states, float *workspace,
+                   size_t workspace_bytes, int b, int h, int64_t n, int d, int e,
+                   int dtype, int seg_len, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LASP_HIP_H */

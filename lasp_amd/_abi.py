@@ -1,0 +1,189 @@
+"""ctypes binding of liblasp_hip.so (the C ABI declared in include/lasp_hip.h).
+
+The library is the only compute path of this package: if it is missing, or a
+tensor is not on a ROCm device, the calls raise -- there is no CPU or eager
+fallback.  Tensors are borrowed as raw device pointers; outputs and workspaces
+come from torch's caching allocator, and work is enqueued on torch's current
+stream, like the Triton launches it replaces
+(lasp/lightning_attention.py:414-429, lasp/lasp_fuse.py:380-399,438-461).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Tuple
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblasp_hip.so")
+_lib = None
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+PATH_GENERIC, PATH_MFMA = 0, 1
+
+_c_void_p = ctypes.c_void_p
+_c_int = ctypes.c_int
+_c_i64 = ctypes.c_int64
+_c_size = ctypes.c_size_t
+
+
+class LaspError(RuntimeError):
+    pass
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Loads the shared library once; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        raise LaspError(
+            f"{_LIB_PATH} is missing: build it with `python -m lasp_amd.build` "
+            "(hipcc --offload-arch=gfx950); lasp_amd has no fallback path"
+        )
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.lasp_abi_version.restype = _c_int
+    lib.lasp_abi_version.argtypes = []
+    lib.lasp_last_error.restype = ctypes.c_char_p
+    lib.lasp_last_error.argtypes = []
+    lib.lasp_plan.restype = _c_int
+    lib.lasp_plan.argtypes = [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                              ctypes.POINTER(_c_int), ctypes.POINTER(_c_int), ctypes.POINTER(_c_size)]
+    lib.lasp_kernel_path.restype = _c_int
+    lib.lasp_kernel_path.argtypes = [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int]
+    lib.lasp_chunk_fwd.restype = _c_int
+    lib.lasp_chunk_fwd.argtypes = [_c_void_p] * 8 + [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
+    lib.lasp_chunk_bwd.restype = _c_int
+    lib.lasp_chunk_bwd.argtypes = [_c_void_p] * 13 + [_c_size, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
+    if lib.lasp_abi_version() != 1:
+        raise LaspError(f"ABI version mismatch: library reports {lib.lasp_abi_version()}, binding expects 1")
+    _lib = lib
+    return lib
+
+
+def _raise(rc: int, what: str):
+    msg = load().lasp_last_error().decode("utf-8", "replace")
+    raise LaspError(f"{what} failed (code {rc}): {msg}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _check_dev(*tensors):
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise LaspError("lasp_amd runs on ROCm devices only; got a tensor on " + str(t.device))
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise LaspError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def _check_state(name, t, b, h, d, e):
+    if t is None:
+        return
+    if t.dtype != torch.float32 or tuple(t.shape) != (b, h, d, e) or not t.is_contiguous():
+        raise LaspError(f"{name} must be a contiguous float32 tensor of shape {(b, h, d, e)}, "
+                        f"got {t.dtype} {tuple(t.shape)}")
+
+
+def plan(b: int, h: int, n: int, d: int, e: int, dtype: torch.dtype, seg_len: int = 0) -> Tuple[int, int, int]:
+    """(seg_len, n_seg, bytes of one segment-state array) for a shape."""
+    lib = load()
+    sl, ns, sb = _c_int(0), _c_int(0), _c_size(0)
+    rc = lib.lasp_plan(b, h, n, d, e, DTYPE_CODE[dtype], seg_len, ctypes.byref(sl), ctypes.byref(ns), ctypes.byref(sb))
+    if rc:
+        _raise(rc, "lasp_plan")
+    return sl.value, ns.value, sb.value
+
+
+def kernel_path(b, h, n, d, e, dtype) -> int:
+    rc = load().lasp_kernel_path(b, h, n, d, e, DTYPE_CODE[dtype])
+    if rc < 0:
+        _raise(rc, "lasp_kernel_path")
+    return rc
+
+
+def _shapes(q, k, v):
+    if q.dim() != 4 or k.shape != q.shape or v.dim() != 4 or v.shape[:3] != q.shape[:3]:
+        raise LaspError(f"expected q,k (b,h,n,d) and v (b,h,n,e); got {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}")
+    if q.dtype not in DTYPE_CODE or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise LaspError(f"q, k, v must share one of float32/bfloat16/float16; got {q.dtype}, {k.dtype}, {v.dtype}")
+    b, h, n, d = q.shape
+    return b, h, n, d, v.shape[-1]
+
+
+def _slopes(s: torch.Tensor, h: int, dev) -> torch.Tensor:
+    if s.numel() != h:
+        raise LaspError(f"need {h} slopes, got a tensor with {s.numel()} elements")
+    return s.detach().to(device=dev, dtype=torch.float32).contiguous()
+
+
+def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
+    """Enqueues the forward of one chunk.  Returns (o, seg_states, seg_len).
+
+    seg_states is the (b, h, n_seg, d, e) float32 array of states entering each
+    segment (None when the call needed none); pass it to chunk_bwd to skip the
+    recompute.
+    """
+    lib = load()
+    dev = _check_dev(q, k, v, kv_in, kv_out)
+    b, h, n, d, e = _shapes(q, k, v)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    s = _slopes(s, h, dev)
+    _check_state("kv_in", kv_in, b, h, d, e)
+    _check_state("kv_out", kv_out, b, h, d, e)
+    seg_len, n_seg, _ = plan(b, h, n, d, e, q.dtype, seg_len)
+    with torch.cuda.device(dev):
+        o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
+        states = None
+        if n_seg > 1 or kv_in is not None or kv_out is not None:
+            states = torch.empty((b, h, n_seg, d, e), dtype=torch.float32, device=dev)
+        rc = lib.lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
+                                o.data_ptr(), _ptr(states), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
+                                torch.cuda.current_stream(dev).cuda_stream)
+    if rc:
+        _raise(rc, "lasp_chunk_fwd")
+    return o, states, seg_len
+
+
+def chunk_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):
+    """Enqueues the backward of one chunk.  Returns (dq, dk, dv)."""
+    lib = load()
+    dev = _check_dev(q, k, v, do, kv_in, dkv_in, dkv_out, kv_seg_states)
+    b, h, n, d, e = _shapes(q, k, v)
+    if do.shape != v.shape or do.dtype != q.dtype:
+        raise LaspError(f"do must match v: {tuple(do.shape)} {do.dtype} vs {tuple(v.shape)} {q.dtype}")
+    q, k, v, do = q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous()
+    s = _slopes(s, h, dev)
+    _check_state("kv_in", kv_in, b, h, d, e)
+    _check_state("dkv_in", dkv_in, b, h, d, e)
+    _check_state("dkv_out", dkv_out, b, h, d, e)
+    seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
+    if kv_seg_states is not None:
+        if (kv_seg_states.dtype != torch.float32 or tuple(kv_seg_states.shape) != (b, h, n_seg, d, e)
+                or not kv_seg_states.is_contiguous()):
+            raise LaspError(f"kv_seg_states must be contiguous float32 {(b, h, n_seg, d, e)}, got "
+                            f"{kv_seg_states.dtype} {tuple(kv_seg_states.shape)}")
+    with torch.cuda.device(dev):
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        n_arrays = 2 if kv_seg_states is None else 1
+        ws = torch.empty((n_arrays * state_bytes // 4,), dtype=torch.float32, device=dev)
+        rc = lib.lasp_chunk_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), _ptr(kv_in),
+                                _ptr(dkv_in), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _ptr(dkv_out),
+                                _ptr(kv_seg_states), ws.data_ptr(), ws.numel() * 4, b, h, n, d, e,
+                                DTYPE_CODE[q.dtype], seg_len, torch.cuda.current_stream(dev).cuda_stream)
+    if rc:
+        _raise(rc, "lasp_chunk_bwd")
+    return dq, dk, dv

@@ -1,0 +1,173 @@
+// C ABI of liblasp_hip.so: argument validation, segment planning and dispatch to
+// the kernel families.  Declarations and the tensor contract: include/lasp_hip.h.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "lasp_common.h"
+
+namespace lasp {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+namespace {
+
+constexpr int kMaxFeature = 128;     // d and e of one launch (the Python wrappers slice d, as
+                                     // lasp/lightning_attention.py:513-519 does)
+constexpr int kSegQuantum = 64;      // segment lengths are multiples of this
+constexpr int64_t kTargetGroups = 512;  // workgroups wanted per launch (2 per CU on 256 CUs)
+constexpr int kMinSeg = 256;
+
+int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
+  if (dtype != LASP_DTYPE_F32 && dtype != LASP_DTYPE_BF16 && dtype != LASP_DTYPE_F16) {
+    set_error("unknown dtype code %d", dtype);
+    return LASP_E_DTYPE;
+  }
+  if (b <= 0 || h <= 0 || n <= 0 || d <= 0 || e <= 0 || d > kMaxFeature || e > kMaxFeature) {
+    set_error("unsupported shape b=%d h=%d n=%lld d=%d e=%d (need b,h,n >= 1 and 1 <= d,e <= %d)", b,
+              h, (long long)n, d, e, kMaxFeature);
+    return LASP_E_SHAPE;
+  }
+  if ((int64_t)b * h > (int64_t)1 << 24) {
+    set_error("b*h = %lld is too large", (long long)b * h);
+    return LASP_E_SHAPE;
+  }
+  return 0;
+}
+
+int default_seg_len(int b, int h, int64_t n) {
+  const int64_t bh = (int64_t)b * h;
+  const int64_t want = (kTargetGroups + bh - 1) / bh;  // segments per (b, h)
+  int64_t len = n / (want > 0 ? want : 1);
+  len = (len / kMinSeg) * kMinSeg;
+  if (len < kMinSeg) len = kMinSeg;
+  return (int)len;
+}
+
+int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
+  int rc = check_shape(b, h, n, d, e, dtype);
+  if (rc) return rc;
+  if (seg_len == 0) seg_len = default_seg_len(b, h, n);
+  if (seg_len < 0 || seg_len % kSegQuantum != 0) {
+    set_error("seg_len=%d must be a positive multiple of %d (or 0 for the default)", seg_len,
+              kSegQuantum);
+    return LASP_E_SEGMENT;
+  }
+  const int64_t n_seg = (n + seg_len - 1) / seg_len;
+  if (n_seg > (1 << 20) || (int64_t)b * h * n_seg > (int64_t)1 << 30) {
+    set_error("too many segments (%lld) for seg_len=%d", (long long)n_seg, seg_len);
+    return LASP_E_SEGMENT;
+  }
+  g->b = b;
+  g->h = h;
+  g->n = n;
+  g->d = d;
+  g->e = e;
+  g->seg_len = seg_len;
+  g->n_seg = (int)n_seg;
+  return 0;
+}
+
+bool mfma_eligible(const Geom &g, int dtype) {
+  return dtype == LASP_DTYPE_BF16 && g.d == 128 && g.e == 128 && g.n % 64 == 0;
+}
+
+size_t state_bytes_of(const Geom &g) {
+  return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.d * g.e;
+}
+
+}  // namespace
+}  // namespace lasp
+
+using namespace lasp;
+
+extern "C" {
+
+int lasp_abi_version(void) { return LASP_ABI_VERSION; }
+
+const char *lasp_last_error(void) { return g_err; }
+
+int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0, int *seg_len,
+              int *n_seg, size_t *state_bytes) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, seg_len_or_0, &g);
+  if (rc) return rc;
+  if (seg_len) *seg_len = g.seg_len;
+  if (n_seg) *n_seg = g.n_seg;
+  if (state_bytes) *state_bytes = state_bytes_of(g);
+  return 0;
+}
+
+int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, 0, &g);
+  if (rc) return rc;
+  return mfma_eligible(g, dtype) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
+}
+
+int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, const float *kv_in,
+                   float *kv_out, void *o, float *seg_states, int b, int h, int64_t n, int d, int e,
+                   int dtype, int seg_len, void *stream) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, seg_len, &g);
+  if (rc) return rc;
+  if (!q || !k || !v || !s || !o) {
+    set_error("lasp_chunk_fwd: q, k, v, s and o must not be NULL");
+    return LASP_E_NULL;
+  }
+  if (!seg_states && (g.n_seg > 1 || kv_in || kv_out)) {
+    set_error("lasp_chunk_fwd: seg_states workspace (%zu bytes) is required for n_seg=%d%s",
+              state_bytes_of(g), g.n_seg, (kv_in || kv_out) ? " with KV in/out" : "");
+    return LASP_E_WORKSPACE;
+  }
+  FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
+  hipStream_t st = (hipStream_t)stream;
+  rc = mfma_eligible(g, dtype) ? mfma_fwd(a, g, st) : generic_fwd(a, g, dtype, st);
+  if (rc > 0) set_error("lasp_chunk_fwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
+  return rc;
+}
+
+int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, const void *d_o,
+                   const float *kv_in, const float *dkv_in, void *dq, void *dk, void *dv,
+                   float *dkv_out, const float *kv_seg_states, float *workspace,
+                   size_t workspace_bytes, int b, int h, int64_t n, int d, int e, int dtype,
+                   int seg_len, void *stream) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, seg_len, &g);
+  if (rc) return rc;
+  if (!q || !k || !v || !s || !d_o || !dq || !dk || !dv) {
+    set_error("lasp_chunk_bwd: q, k, v, s, do, dq, dk and dv must not be NULL");
+    return LASP_E_NULL;
+  }
+  const size_t one = state_bytes_of(g);
+  const bool need_kv = !kv_seg_states && (g.n_seg > 1 || kv_in);
+  const bool need_dkv = g.n_seg > 1 || dkv_in || dkv_out;
+  const size_t need = one * ((need_kv ? 1 : 0) + (need_dkv ? 1 : 0));
+  if (need && (!workspace || workspace_bytes < need)) {
+    set_error("lasp_chunk_bwd: workspace of %zu bytes required, got %zu", need,
+              workspace ? workspace_bytes : (size_t)0);
+    return LASP_E_WORKSPACE;
+  }
+  BwdArgs a{q,  k,  v,       s,
+            d_o, kv_in, dkv_in, dq,
+            dk, dv, dkv_out, kv_seg_states,
+            nullptr, nullptr};
+  float *wp = workspace;
+  if (need_dkv) {
+    a.ws_dkv = wp;
+    wp += one / sizeof(float);
+  }
+  if (need_kv) a.ws_kv = wp;
+  hipStream_t st = (hipStream_t)stream;
+  rc = mfma_eligible(g, dtype) ? mfma_bwd(a, g, st) : generic_bwd(a, g, dtype, st);
+  if (rc > 0) set_error("lasp_chunk_bwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,96 @@
+// Shared definitions for the gfx950 kernels behind the C ABI in include/lasp_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "lasp_hip.h"
+
+namespace lasp {
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+__device__ __forceinline__ float bf16_bits_to_f32(bf16_t x) {
+  return __uint_as_float(((uint32_t)x) << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ bf16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+struct bf16_tag {
+  bf16_t bits;
+};
+
+template <class T>
+struct elem;
+template <>
+struct elem<float> {
+  static __device__ __forceinline__ float load(const float *p) { return *p; }
+  static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <>
+struct elem<bf16_tag> {
+  static __device__ __forceinline__ float load(const bf16_tag *p) {
+    return bf16_bits_to_f32(p->bits);
+  }
+  static __device__ __forceinline__ void store(bf16_tag *p, float v) {
+    p->bits = f32_to_bf16_bits(v);
+  }
+};
+template <>
+struct elem<_Float16> {
+  static __device__ __forceinline__ float load(const _Float16 *p) { return (float)*p; }
+  static __device__ __forceinline__ void store(_Float16 *p, float v) { *p = (_Float16)v; }
+};
+
+// One chunk's geometry, passed by value to every kernel.
+struct Geom {
+  int b, h;
+  int64_t n;    // tokens in the chunk
+  int d, e;     // feature sizes of q/k and v/o
+  int seg_len;  // tokens per segment (multiple of 64)
+  int n_seg;    // ceil(n / seg_len)
+};
+
+// Host-side launchers (each returns a hipError_t as int, or a negative LASP_E_*).
+struct FwdArgs {
+  const void *q, *k, *v;
+  const float *s;
+  const float *kv_in;
+  float *kv_out;
+  void *o;
+  float *seg_states;
+};
+struct BwdArgs {
+  const void *q, *k, *v;
+  const float *s;
+  const void *d_o;
+  const float *kv_in, *dkv_in;
+  void *dq, *dk, *dv;
+  float *dkv_out;
+  const float *kv_seg_states;  // may be NULL
+  float *ws_kv;                // used when kv_seg_states is NULL
+  float *ws_dkv;
+};
+
+int generic_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st);
+int generic_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st);
+int mfma_fwd(const FwdArgs &a, const Geom &g, hipStream_t st);
+int mfma_bwd(const BwdArgs &a, const Geom &g, hipStream_t st);
+
+// The decayed scan over segment states is shared by both kernel families.
+//   forward  (reverse = 0): states[seg] <- state entering segment seg from the
+//             left (segment 0: carry_in or 0); carry_out <- state after the chunk
+//   reverse  (reverse = 1): states[seg] <- state entering segment seg from the
+//             right (last segment: carry_in or 0); carry_out <- state before the chunk
+int launch_segment_scan(float *states, const float *carry_in, float *carry_out,
+                        const float *s, const Geom &g, int reverse, hipStream_t st);
+
+void set_error(const char *fmt, ...);
+
+}  // namespace lasp

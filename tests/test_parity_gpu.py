@@ -1,0 +1,107 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle.
+
+Error metric: max|x - ref| / max|ref| per output tensor, ref = fp64 oracle on the
+same rounded inputs.  Tolerances: 1e-3 for fp32 I/O, 2e-2 for bf16 / fp16 I/O.
+"""
+import pytest
+import torch
+
+from oracle import lasp_oracle as O
+from tests.helpers import TOL, check, make_inputs, oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def run_abi(inp, s, dev, seg_len=0, cache=False):
+    """One chunk forward + backward through lasp_amd._abi (ctypes -> liblasp_hip.so)."""
+    from lasp_amd import _abi
+
+    t = {k_: (x.to(dev) if x is not None else None) for k_, x in inp.items()}
+    kv_out = torch.empty_like(t["kv"]) if t["kv"] is not None else None
+    dkv_out = torch.empty_like(t["dkv"]) if t["dkv"] is not None else None
+    o, states, sl = _abi.chunk_fwd(t["q"], t["k"], t["v"], s, kv_in=t["kv"], kv_out=kv_out, seg_len=seg_len)
+    dq, dk, dv = _abi.chunk_bwd(t["q"], t["k"], t["v"], s, t["do"], kv_in=t["kv"], dkv_in=t["dkv"],
+                                dkv_out=dkv_out, kv_seg_states=states if cache else None, seg_len=sl)
+    torch.cuda.synchronize()
+    return dict(o=o, kv_out=kv_out, dq=dq, dk=dk, dv=dv, dkv_out=dkv_out)
+
+
+def test_library_loaded_and_path_selection(gpu_device):
+    from lasp_amd import _abi
+
+    lib = _abi.load()
+    assert lib.lasp_abi_version() == 1
+    assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_GENERIC
+
+
+@pytest.mark.parametrize("state", [False, True])
+@pytest.mark.parametrize("shape", [
+    (1, 2, 64, 32, 32, 0), (2, 3, 200, 64, 32, 0), (1, 2, 7, 16, 48, 0),
+    (1, 2, 1024, 128, 128, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0),
+])
+def test_generic_fp32_small(gpu_device, shape, state):
+    b, h, n, d, e, seg = shape
+    inp = make_inputs(b, h, n, d, e, torch.float32, seed=n + d, state=state, state_std=1.0)
+    s = O.slopes_baseline(h)
+    got = run_abi(inp, s, gpu_device, seg_len=seg)
+    check(got, oracle(inp, s), 1e-3 if n > 64 else 2e-4, what=f"fp32 {shape} state={state}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_generic_low_precision_io(gpu_device, dtype):
+    # e != d keeps these on the generic kernels (the reference test shape has e = 64)
+    inp = make_inputs(2, 12, 512, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    s = O.slopes_alibi(12)
+    got = run_abi(inp, s, gpu_device)
+    check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
+
+
+def test_special_slopes_zero_and_huge(gpu_device):
+    inp = make_inputs(1, 2, 300, 32, 32, torch.float32, seed=5, state=True, state_std=1.0)
+    s = torch.tensor([0.0, 50.0])
+    got = run_abi(inp, s, gpu_device)
+    assert all(torch.isfinite(v_).all() for v_ in got.values())
+    check(got, oracle(inp, s), 1e-3, what="s in {0, 50}")
+
+
+def test_cached_states_equal_recompute(gpu_device):
+    inp = make_inputs(1, 4, 1024, 128, 128, torch.float32, seed=6, state=True, state_std=1.0)
+    s = O.slopes_baseline(4)
+    a = run_abi(inp, s, gpu_device, seg_len=256, cache=False)
+    c = run_abi(inp, s, gpu_device, seg_len=256, cache=True)
+    for name in ("dq", "dk", "dv", "dkv_out"):
+        assert torch.equal(a[name], c[name]), name
+
+
+def test_segment_length_does_not_change_result(gpu_device):
+    inp = make_inputs(1, 2, 1536, 64, 64, torch.float32, seed=7, state=True, state_std=1.0)
+    s = O.slopes_baseline(2)
+    ref = oracle(inp, s)
+    for seg in (64, 512, 2048):
+        check(run_abi(inp, s, gpu_device, seg_len=seg), ref, 1e-3, what=f"seg_len={seg}")
+
+
+def test_config0_fp32_full(gpu_device):
+    """BASELINE config 0: b=2 n=2048 h=12 d=128 fp32, no incoming state."""
+    inp = make_inputs(2, 12, 2048, 128, 128, torch.float32, seed=0, state=False)
+    s = O.slopes_baseline(12)
+    got = run_abi(inp, s, gpu_device)
+    check(got, oracle(inp, s), 1e-3, what="config 0")
+
+
+def test_argument_errors(gpu_device):
+    from lasp_amd import _abi
+
+    q = torch.zeros(1, 1, 64, 256, device=gpu_device)
+    with pytest.raises(_abi.LaspError, match="unsupported shape"):
+        _abi.chunk_fwd(q, q, q, torch.ones(1))
+    q = torch.zeros(1, 1, 64, 64, device=gpu_device)
+    with pytest.raises(_abi.LaspError, match="seg_len"):
+        _abi.chunk_fwd(q, q, q, torch.ones(1), seg_len=100)
+    with pytest.raises(_abi.LaspError, match="slopes"):
+        _abi.chunk_fwd(q, q, q, torch.ones(3))
+    with pytest.raises(_abi.LaspError, match="ROCm"):
+        _abi.chunk_fwd(q.cpu(), q.cpu(), q.cpu(), torch.ones(1))
