@@ -105,3 +105,45 @@ def test_argument_errors(gpu_device):
         _abi.chunk_fwd(q, q, q, torch.ones(3))
     with pytest.raises(_abi.LaspError, match="ROCm"):
         _abi.chunk_fwd(q.cpu(), q.cpu(), q.cpu(), torch.ones(1))
+
+
+# ---------------------------------------------------------------- bf16 MFMA kernels (d = e = 128)
+@pytest.mark.parametrize("state", [False, True])
+@pytest.mark.parametrize("b,h,n,seg", [
+    (1, 1, 64, 0), (1, 2, 128, 64), (1, 2, 256, 0), (2, 3, 512, 128), (1, 4, 1024, 256), (1, 2, 2048, 2048),
+])
+def test_mfma_bf16(gpu_device, b, h, n, seg, state):
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(b, h, n, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
+    inp = make_inputs(b, h, n, 128, 128, torch.bfloat16, seed=n + h, state=state, state_std=1.0)
+    s = O.slopes_baseline(h) if h > 1 else torch.tensor([0.05])
+    got = run_abi(inp, s, gpu_device, seg_len=seg)
+    check(got, oracle(inp, s), 2e-2, what=f"mfma b={b} h={h} n={n} seg={seg} state={state}")
+
+
+def test_mfma_special_slopes(gpu_device):
+    inp = make_inputs(1, 3, 512, 128, 128, torch.bfloat16, seed=11, state=True, state_std=1.0)
+    s = torch.tensor([0.0, 1.0, 30.0])
+    got = run_abi(inp, s, gpu_device, seg_len=128)
+    assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
+    check(got, oracle(inp, s), 2e-2, what="mfma s in {0, 1, 30}")
+
+
+def test_mfma_inter_path_in_isolation(gpu_device):
+    # K = V = 0 leaves O = diag(l^i) Q KV_in and dQ = diag(l^i) dO KV_in^T: the state operand alone
+    inp = make_inputs(1, 2, 256, 128, 128, torch.bfloat16, seed=12, state=True, state_std=1.0)
+    inp["k"].zero_()
+    inp["v"].zero_()
+    s = torch.tensor([0.02, 0.3])
+    got = run_abi(inp, s, gpu_device, seg_len=128)
+    check(got, oracle(inp, s), 2e-2, what="mfma inter only")
+
+
+def test_mfma_cached_states_equal_recompute(gpu_device):
+    inp = make_inputs(1, 4, 1024, 128, 128, torch.bfloat16, seed=13, state=True, state_std=1.0)
+    s = O.slopes_baseline(4)
+    a = run_abi(inp, s, gpu_device, seg_len=256, cache=False)
+    c = run_abi(inp, s, gpu_device, seg_len=256, cache=True)
+    for name in ("dq", "dk", "dv", "dkv_out"):
+        assert torch.equal(a[name], c[name]), name
