@@ -112,6 +112,23 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
                    size_t workspace_bytes, int b, int h, int64_t n, int d, int e,
                    int dtype, int seg_len, void *stream);
 
+/*
+ * Measurement hook (no counterpart in the reference, which times nothing).
+ * Between lasp_profile_begin and lasp_profile_end every kernel the library
+ * launches is bracketed by two hipEvents on its launch stream (at most
+ * max_launches of them; later launches go untimed).  lasp_profile_end waits for
+ * the recorded events and returns, per kernel class, the summed duration in
+ * milliseconds and the number of launches (arrays of LASP_KERNEL_CLASSES
+ * entries; either may be NULL).  One profile at a time, one thread.
+ */
+#define LASP_KERNEL_CLASSES 4
+#define LASP_KC_APPLY 0   /* la_apply: the block sweep producing O, dQ, dK or dV */
+#define LASP_KC_STATE 1   /* la_seg_state: per-segment state pre-pass */
+#define LASP_KC_SCAN 2    /* decayed scan over segment states */
+#define LASP_KC_GENERIC 3 /* any kernel of the generic fp32-FMA family */
+int lasp_profile_begin(int max_launches);
+int lasp_profile_end(double *ms_per_class, int *launches_per_class);
+
 #ifdef __cplusplus
 }
 #endif

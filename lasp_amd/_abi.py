@@ -59,6 +59,10 @@ def load() -> ctypes.CDLL:
     lib.lasp_chunk_fwd.argtypes = [_c_void_p] * 8 + [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
     lib.lasp_chunk_bwd.restype = _c_int
     lib.lasp_chunk_bwd.argtypes = [_c_void_p] * 13 + [_c_size, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
+    lib.lasp_profile_begin.restype = _c_int
+    lib.lasp_profile_begin.argtypes = [_c_int]
+    lib.lasp_profile_end.restype = _c_int
+    lib.lasp_profile_end.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_c_int)]
     if lib.lasp_abi_version() != 1:
         raise LaspError(f"ABI version mismatch: library reports {lib.lasp_abi_version()}, binding expects 1")
     _lib = lib
@@ -111,6 +115,26 @@ def kernel_path(b, h, n, d, e, dtype) -> int:
     if rc < 0:
         _raise(rc, "lasp_kernel_path")
     return rc
+
+
+KERNEL_CLASSES = ("apply", "state", "scan", "generic")
+
+
+def profile_begin(max_launches: int = 4096) -> None:
+    """Starts bracketing every kernel launch of the library with HIP events."""
+    rc = load().lasp_profile_begin(max_launches)
+    if rc:
+        _raise(rc, "lasp_profile_begin")
+
+
+def profile_end() -> dict:
+    """Waits for the bracketed launches; {class: (total_ms, launches)}."""
+    ms = (ctypes.c_double * 4)()
+    cnt = (_c_int * 4)()
+    rc = load().lasp_profile_end(ms, cnt)
+    if rc:
+        _raise(rc, "lasp_profile_end")
+    return {name: (ms[i], cnt[i]) for i, name in enumerate(KERNEL_CLASSES)}
 
 
 def _shapes(q, k, v):

@@ -16,6 +16,24 @@ void set_error(const char *fmt, ...) {
   va_end(ap);
 }
 
+// ---- per-kernel timing -------------------------------------------------------
+struct ProfEntry {
+  int cls;
+  hipEvent_t start, stop;
+};
+static ProfEntry *g_prof = nullptr;  // non-NULL while a profile is open
+static int g_prof_cap = 0, g_prof_used = 0;
+
+ProfScope::ProfScope(int kernel_class, hipStream_t st) : slot(-1), stream(st) {
+  if (!g_prof || g_prof_used >= g_prof_cap) return;
+  slot = g_prof_used++;
+  g_prof[slot].cls = kernel_class;
+  (void)hipEventRecord(g_prof[slot].start, stream);
+}
+ProfScope::~ProfScope() {
+  if (slot >= 0) (void)hipEventRecord(g_prof[slot].stop, stream);
+}
+
 namespace {
 
 constexpr int kMaxFeature = 128;     // d and e of one launch (the Python wrappers slice d, as
@@ -92,6 +110,59 @@ extern "C" {
 int lasp_abi_version(void) { return LASP_ABI_VERSION; }
 
 const char *lasp_last_error(void) { return g_err; }
+
+int lasp_profile_begin(int max_launches) {
+  if (g_prof) {
+    set_error("lasp_profile_begin: a profile is already open");
+    return LASP_E_SHAPE;
+  }
+  if (max_launches <= 0 || max_launches > (1 << 20)) {
+    set_error("lasp_profile_begin: max_launches=%d out of range", max_launches);
+    return LASP_E_SHAPE;
+  }
+  ProfEntry *p = new ProfEntry[max_launches];
+  for (int i = 0; i < max_launches; ++i) {
+    hipError_t e1 = hipEventCreate(&p[i].start), e2 = hipEventCreate(&p[i].stop);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("lasp_profile_begin: hipEventCreate failed");
+      return (int)(e1 != hipSuccess ? e1 : e2);
+    }
+  }
+  g_prof_cap = max_launches;
+  g_prof_used = 0;
+  g_prof = p;
+  return 0;
+}
+
+int lasp_profile_end(double *ms_per_class, int *launches_per_class) {
+  if (!g_prof) {
+    set_error("lasp_profile_end: no profile is open");
+    return LASP_E_SHAPE;
+  }
+  ProfEntry *p = g_prof;
+  g_prof = nullptr;
+  for (int c = 0; c < KC_COUNT; ++c) {
+    if (ms_per_class) ms_per_class[c] = 0.0;
+    if (launches_per_class) launches_per_class[c] = 0;
+  }
+  int rc = 0;
+  for (int i = 0; i < g_prof_used; ++i) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(p[i].stop);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, p[i].start, p[i].stop);
+    if (e != hipSuccess) rc = (int)e;
+    if (ms_per_class) ms_per_class[p[i].cls] += ms;
+    if (launches_per_class) launches_per_class[p[i].cls] += 1;
+  }
+  for (int i = 0; i < g_prof_cap; ++i) {
+    (void)hipEventDestroy(p[i].start);
+    (void)hipEventDestroy(p[i].stop);
+  }
+  delete[] p;
+  g_prof_cap = g_prof_used = 0;
+  if (rc) set_error("lasp_profile_end: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
+  return rc;
+}
 
 int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0, int *seg_len,
               int *n_seg, size_t *state_bytes) {

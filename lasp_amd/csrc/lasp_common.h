@@ -93,4 +93,14 @@ int launch_segment_scan(float *states, const float *carry_in, float *carry_out,
 
 void set_error(const char *fmt, ...);
 
+// Optional per-kernel timing (lasp_profile_begin / lasp_profile_end): while a
+// profile is open every kernel launch is bracketed by two events on its stream.
+enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_COUNT = 4 };
+struct ProfScope {
+  ProfScope(int kernel_class, hipStream_t st);
+  ~ProfScope();
+  int slot;
+  hipStream_t stream;
+};
+
 }  // namespace lasp

@@ -364,11 +364,15 @@ int fwd_t(const FwdArgs &a, const Geom &g, hipStream_t st) {
   if (need_states) {
     const size_t lds = sizeof(float) * (GB * ldd + GB * lde + d * lde + 2 * GB);
     if ((rc = set_lds(generic_seg_state<T>, lds))) return rc;
-    generic_seg_state<T><<<grid, NT, lds, st>>>((const T *)a.k, (const T *)a.v, a.s, a.seg_states, g, 0);
+    {
+      ProfScope prof(KC_GENERIC, st);
+      generic_seg_state<T><<<grid, NT, lds, st>>>((const T *)a.k, (const T *)a.v, a.s, a.seg_states, g, 0);
+    }
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
   const size_t lds = sizeof(float) * (2 * GB * ldd + GB * lde + GB * LDS_S + d * lde + 2 * GB);
   if ((rc = set_lds(generic_fwd_apply<T>, lds))) return rc;
+  ProfScope prof(KC_GENERIC, st);
   generic_fwd_apply<T><<<grid, NT, lds, st>>>((const T *)a.q, (const T *)a.k, (const T *)a.v, a.s,
                                               need_states ? a.seg_states : nullptr, (T *)a.o, g);
   return (int)hipGetLastError();
@@ -384,19 +388,26 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
 
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    generic_seg_state<T><<<grid, NT, lds_state, st>>>((const T *)a.k, (const T *)a.v, a.s, a.ws_kv, g, 0);
+    {
+      ProfScope prof(KC_GENERIC, st);
+      generic_seg_state<T><<<grid, NT, lds_state, st>>>((const T *)a.k, (const T *)a.v, a.s, a.ws_kv, g, 0);
+    }
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    generic_seg_state<T><<<grid, NT, lds_state, st>>>((const T *)a.q, (const T *)a.d_o, a.s, a.ws_dkv, g, 1);
+    {
+      ProfScope prof(KC_GENERIC, st);
+      generic_seg_state<T><<<grid, NT, lds_state, st>>>((const T *)a.q, (const T *)a.d_o, a.s, a.ws_dkv, g, 1);
+    }
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
   {
     const size_t lds = sizeof(float) * (2 * GB * lde + GB * ldd + GB * LDS_S + d * lde + 2 * GB);
     if ((rc = set_lds(generic_bwd_dq<T>, lds))) return rc;
+    ProfScope prof(KC_GENERIC, st);
     generic_bwd_dq<T><<<grid, NT, lds, st>>>((const T *)a.k, (const T *)a.v, (const T *)a.d_o, a.s,
                                              kv_states, (T *)a.dq, g);
   }
@@ -404,6 +415,7 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
     const size_t lds =
         sizeof(float) * (2 * GB * ldd + 2 * GB * lde + 2 * GB * LDS_S + d * lde + 2 * GB);
     if ((rc = set_lds(generic_bwd_dkdv<T>, lds))) return rc;
+    ProfScope prof(KC_GENERIC, st);
     generic_bwd_dkdv<T><<<grid, NT, lds, st>>>((const T *)a.q, (const T *)a.k, (const T *)a.v,
                                                (const T *)a.d_o, a.s, dkv_states, (T *)a.dk,
                                                (T *)a.dv, g);
@@ -417,6 +429,7 @@ int launch_segment_scan(float *states, const float *carry_in, float *carry_out, 
                         const Geom &g, int reverse, hipStream_t st) {
   const int64_t total = (int64_t)g.b * g.h * g.d * g.e;
   const unsigned grid = (unsigned)((total + 255) / 256);
+  ProfScope prof(KC_SCAN, st);
   segment_scan_kernel<<<grid, 256, 0, st>>>(states, carry_in, carry_out, s, g, reverse);
   return (int)hipGetLastError();
 }

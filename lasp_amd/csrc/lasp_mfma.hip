@@ -412,6 +412,7 @@ int launch_apply(const void *x, const void *y, const void *z, const float *s, co
   int rc = raise_lds(la_apply<REV, TRANS>);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_APPLY, st);
   la_apply<REV, TRANS><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
                                                       (const bf16_t *)z, s, states, (bf16_t *)out, g);
   return (int)hipGetLastError();
@@ -421,6 +422,7 @@ template <bool REV>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_STATE, st);
   la_seg_state<REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g);
   return (int)hipGetLastError();
 }

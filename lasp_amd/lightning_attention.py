@@ -15,7 +15,9 @@ class LightningAttention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, s):
-        return ChunkFunction.forward(ctx, q, k, v, s, None, None, False, False)
+        # the per-segment states (64 KiB per (b, h, segment)) are kept for backward:
+        # cheaper than re-reading K and V to rebuild them
+        return ChunkFunction.forward(ctx, q, k, v, s, None, None, True, False)
 
     @staticmethod
     def backward(ctx, do):
@@ -30,4 +32,4 @@ def lightning_attn(q, k, v, ed):
     d = q.shape[-1]
     if d <= 128:
         return lightning_attn_(q, k, v, ed)
-    return run_sliced(q, k, v, ed, None, None, False, False)
+    return run_sliced(q, k, v, ed, None, None, True, False)

@@ -1,0 +1,111 @@
+"""CPU-side checks of the C ABI: the library loads, exports every function that
+include/lasp_hip.h declares, and its host-only entry points (planning, argument
+validation) behave.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "lasp_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from lasp_amd import _abi
+
+    if not os.path.exists(_abi.lib_path()):
+        from lasp_amd import build
+
+        build.build(verbose=False)
+    return _abi.load()
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"\b(lasp_[a-z_0-9]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared_functions()
+    for must in ("lasp_abi_version", "lasp_last_error", "lasp_plan", "lasp_kernel_path", "lasp_chunk_fwd",
+                 "lasp_chunk_bwd", "lasp_profile_begin", "lasp_profile_end"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(lib):
+    for name in _declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in lasp_hip.h but not exported"
+    assert lib.lasp_abi_version() == 1
+
+
+def test_plan_defaults_and_overrides(lib):
+    from lasp_amd import _abi
+
+    # headline shape: 16 (b,h) pairs -> 32 segments of 2048 tokens = 512 workgroups
+    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16) == (2048, 32, 16 * 32 * 128 * 128 * 4)
+    # short chunk: never below 256 tokens per segment
+    assert _abi.plan(2, 12, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
+    # ragged n: last segment shorter
+    assert _abi.plan(1, 1, 300, 64, 32, torch.float32, 64)[:2] == (64, 5)
+    assert _abi.plan(1, 1, 300, 64, 32, torch.float32, 64)[2] == 5 * 64 * 32 * 4
+    # many heads: one segment covers the chunk
+    sl, ns, _ = _abi.plan(8, 128, 4096, 128, 128, torch.bfloat16)
+    assert ns == 1 and sl >= 4096
+
+
+def test_plan_rejects_bad_arguments(lib):
+    from lasp_amd import _abi
+
+    with pytest.raises(_abi.LaspError, match="unsupported shape"):
+        _abi.plan(1, 1, 64, 129, 64, torch.float32)
+    with pytest.raises(_abi.LaspError, match="unsupported shape"):
+        _abi.plan(1, 1, 0, 64, 64, torch.float32)
+    with pytest.raises(_abi.LaspError, match="seg_len"):
+        _abi.plan(1, 1, 640, 64, 64, torch.float32, 96)
+    rc = lib.lasp_plan(1, 1, 64, 64, 64, 7, 0, None, None, None)
+    assert rc == -3 and b"dtype" in lib.lasp_last_error()
+
+
+def test_kernel_path_selection(lib):
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.float16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.float32) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65500, 128, 128, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_GENERIC
+
+
+def test_null_and_workspace_errors_need_no_gpu(lib):
+    # argument validation happens before any HIP call
+    rc = lib.lasp_chunk_fwd(None, None, None, None, None, None, None, None, 1, 1, 64, 64, 64, 0, 0, None)
+    assert rc == -1
+    one = ctypes.c_void_p(16)  # never dereferenced: validation fails first
+    rc = lib.lasp_chunk_fwd(one, one, one, one, None, None, one, None, 1, 1, 1024, 64, 64, 0, 256, None)
+    assert rc == -5 and b"seg_states" in lib.lasp_last_error()
+    rc = lib.lasp_chunk_bwd(one, one, one, one, one, None, None, one, one, one, None, None, None, 0,
+                            1, 1, 1024, 64, 64, 0, 256, None)
+    assert rc == -5 and b"workspace" in lib.lasp_last_error()
+
+
+def test_product_path_refuses_cpu_tensors(lib):
+    import lasp_amd
+    from lasp_amd import _abi
+
+    x = torch.zeros(1, 1, 64, 64)
+    with pytest.raises(_abi.LaspError, match="ROCm devices only"):
+        lasp_amd.lightning_attn(x, x, x, torch.ones(1))
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "lasp_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, f"{f} mentions the oracle"

@@ -1,0 +1,122 @@
+"""The public operators (autograd Functions + loopback state passing) against the
+oracle, at the BASELINE configurations or scaled-down versions of them.
+
+Tolerance: max|x - ref| / max|ref| <= 2e-2 for bf16 I/O (1e-3 for fp32)."""
+import pytest
+import torch
+
+from oracle import lasp_oracle as O
+from tests.helpers import make_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def _single_pass(fn_inputs, s, dev):
+    import lasp_amd
+
+    q, k, v = [fn_inputs[x].to(dev).requires_grad_(True) for x in ("q", "k", "v")]
+    o = lasp_amd.lightning_attn(q, k, v, s.to(dev))
+    o.backward(fn_inputs["do"].to(dev))
+    torch.cuda.synchronize()
+    return dict(o=o.detach(), dq=q.grad, dk=k.grad, dv=v.grad)
+
+
+def _chain(op_name, inp, s, dev, chunks):
+    """Plays sequence-parallel ranks 0..C-1 on one device through the loopback."""
+    import lasp_amd
+
+    op = getattr(lasp_amd, op_name)
+    b, h, n, d = inp["q"].shape
+    e = inp["v"].shape[-1]
+    step = n // chunks
+    lasp_amd.destroy_parallel_groups()
+    lasp_amd.initialize_lasp(1, chunks)
+    KV = torch.empty(b, h, d, e, device=dev)
+    DKV = torch.empty(b, h, d, e, device=dev)
+    outs, leaves = [], []
+    sd = s.to(dev)
+    try:
+        for c in range(chunks):
+            lasp_amd.set_sequence_parallel_rank(c)
+            sl = slice(c * step, (c + 1) * step)
+            qc, kc, vc = [inp[x][:, :, sl].to(dev).requires_grad_(True) for x in ("q", "k", "v")]
+            if op_name == "lasp_naive":
+                o = op(qc, kc, vc, sd)
+            elif op_name == "lasp_cache":
+                o = op(qc, kc, vc, sd, torch.arange(step, device=dev), KV, DKV)
+            else:
+                o = op(qc, kc, vc, sd, KV, DKV)
+            outs.append(o)
+            leaves.append((qc, kc, vc))
+        for c in reversed(range(chunks)):
+            sl = slice(c * step, (c + 1) * step)
+            outs[c].backward(inp["do"][:, :, sl].to(dev))
+        torch.cuda.synchronize()
+        assert lasp_amd.loopback_pending() == []
+    finally:
+        lasp_amd.destroy_parallel_groups()
+    return dict(
+        o=torch.cat([o.detach() for o in outs], 2),
+        dq=torch.cat([l[0].grad for l in leaves], 2),
+        dk=torch.cat([l[1].grad for l in leaves], 2),
+        dv=torch.cat([l[2].grad for l in leaves], 2),
+    )
+
+
+def _errs(got, ref):
+    return {name: O.rel_err(got[name], ref[name]) for name in ("o", "dq", "dk", "dv")}
+
+
+@pytest.mark.parametrize("op_name", ["lasp_fuse", "lasp_fuse_parallel", "lasp_naive", "lasp_cache"])
+def test_chain_matches_single_pass_and_oracle_small(gpu_device, op_name):
+    # the reference's own test shape, e = 64 (tests/test.py:95), sp = 4
+    inp = make_inputs(2, 12, 2048, 128, 64, torch.bfloat16, seed=21, state=False)
+    s = O.slopes_alibi(12)
+    ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s, inp["do"], dtype=torch.float64)
+    got = _chain(op_name, inp, s, gpu_device, chunks=4)
+    e = _errs(got, ref)
+    assert max(e.values()) <= 2e-2, (op_name, e)
+    sp = _single_pass(inp, s, gpu_device)
+    e2 = _errs(got, {k_: v_.cpu() for k_, v_ in sp.items()})
+    assert max(e2.values()) <= 2e-2, (op_name, e2)
+
+
+def test_config1_chunk_chain_bf16(gpu_device):
+    """BASELINE config 1: b=2 h=12 d=128, n=16384 as 8 chunks of 2048 with KV / DKV carry."""
+    inp = make_inputs(2, 12, 16384, 128, 128, torch.bfloat16, seed=1, state=False)
+    s = O.slopes_baseline(12)
+    ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s, inp["do"], dtype=torch.float32)
+    for op_name in ("lasp_fuse", "lasp_fuse_parallel"):
+        got = _chain(op_name, inp, s, gpu_device, chunks=8)
+        e = _errs(got, ref)
+        assert max(e.values()) <= 2e-2, (op_name, "vs oracle", e)
+        sp = _single_pass(inp, s, gpu_device)
+        e2 = _errs(got, {k_: v_.cpu() for k_, v_ in sp.items()})
+        assert max(e2.values()) <= 2e-2, (op_name, "vs single pass", e2)
+
+
+def test_lightning_attn_fp32_and_wide_heads(gpu_device):
+    import lasp_amd
+
+    # d = 192 > 128 goes through the feature-slicing wrapper (two launches, outputs added)
+    inp = make_inputs(1, 3, 300, 192, 64, torch.float32, seed=22, state=False)
+    s = O.slopes_alibi(3)
+    ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s, inp["do"], dtype=torch.float64)
+    got = _single_pass(inp, s, gpu_device)
+    e = _errs(got, ref)
+    assert max(e.values()) <= 1e-3, e
+
+
+def test_loopback_recv_without_send_raises(gpu_device):
+    import lasp_amd
+
+    lasp_amd.destroy_parallel_groups()
+    lasp_amd.initialize_lasp(1, 2)
+    try:
+        lasp_amd.set_sequence_parallel_rank(1)  # rank 1 runs before rank 0 sent anything
+        x = torch.zeros(1, 1, 64, 64, device=gpu_device, dtype=torch.bfloat16)
+        KV = torch.empty(1, 1, 64, 64, device=gpu_device)
+        with pytest.raises(RuntimeError, match="nothing was sent"):
+            lasp_amd.lasp_fuse(x, x, x, torch.ones(1), KV, torch.empty_like(KV))
+    finally:
+        lasp_amd.destroy_parallel_groups()
