@@ -121,11 +121,12 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
  * milliseconds and the number of launches (arrays of LASP_KERNEL_CLASSES
  * entries; either may be NULL).  One profile at a time, one thread.
  */
-#define LASP_KERNEL_CLASSES 4
-#define LASP_KC_APPLY 0   /* la_apply: the block sweep producing O, dQ, dK or dV */
+#define LASP_KERNEL_CLASSES 5
+#define LASP_KC_APPLY 0   /* la_apply: the block sweep producing O */
 #define LASP_KC_STATE 1   /* la_seg_state: per-segment state pre-pass */
 #define LASP_KC_SCAN 2    /* decayed scan over segment states */
 #define LASP_KC_GENERIC 3 /* any kernel of the generic fp32-FMA family */
+#define LASP_KC_BWD3 4    /* la_bwd3: dQ, dK and dV block sweeps in one launch */
 int lasp_profile_begin(int max_launches);
 int lasp_profile_end(double *ms_per_class, int *launches_per_class);
 

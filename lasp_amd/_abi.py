@@ -117,7 +117,7 @@ def kernel_path(b, h, n, d, e, dtype) -> int:
     return rc
 
 
-KERNEL_CLASSES = ("apply", "state", "scan", "generic")
+KERNEL_CLASSES = ("apply", "state", "scan", "generic", "bwd3")
 
 
 def profile_begin(max_launches: int = 4096) -> None:
@@ -129,8 +129,8 @@ def profile_begin(max_launches: int = 4096) -> None:
 
 def profile_end() -> dict:
     """Waits for the bracketed launches; {class: (total_ms, launches)}."""
-    ms = (ctypes.c_double * 4)()
-    cnt = (_c_int * 4)()
+    ms = (ctypes.c_double * len(KERNEL_CLASSES))()
+    cnt = (_c_int * len(KERNEL_CLASSES))()
     rc = load().lasp_profile_end(ms, cnt)
     if rc:
         _raise(rc, "lasp_profile_end")

@@ -95,7 +95,7 @@ void set_error(const char *fmt, ...);
 
 // Optional per-kernel timing (lasp_profile_begin / lasp_profile_end): while a
 // profile is open every kernel launch is bracketed by two events on its stream.
-enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_COUNT = 4 };
+enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_BWD3 = 4, KC_COUNT = 5 };
 struct ProfScope {
   ProfScope(int kernel_class, hipStream_t st);
   ~ProfScope();

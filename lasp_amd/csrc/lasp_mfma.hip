@@ -34,6 +34,10 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+// native vector types (HIP's u32x4 / u32x2 structs copy through memcpy, which can pin
+// a register array to scratch memory)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef float float2_t __attribute__((ext_vector_type(2)));
 
 constexpr int F = 128;      // feature size (d = e)
@@ -57,26 +61,59 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 
 union Frag {
   bf16x8 v;
-  uint4 q;
-  uint2 h[2];
+  u32x4 q;
+  u32x2 h[2];
   uint32_t w[4];
 };
 
 __device__ __forceinline__ bf16x8 lds16(const char *p) { return *reinterpret_cast<const bf16x8 *>(p); }
 
 // element x (0..7) of a 16-byte group of bf16, widened to fp32
-__device__ __forceinline__ float bf_elem(const uint4 &q, int x) {
+__device__ __forceinline__ float bf_elem(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
   return __uint_as_float((x & 1) ? (w & 0xffff0000u) : (w << 16));
 }
-__device__ __forceinline__ uint32_t bf_bits(const uint4 &q, int x) {
+__device__ __forceinline__ uint32_t bf_bits(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
   return (x & 1) ? (w >> 16) : (w & 0xffffu);
 }
 
-// byte offset of 16-byte granule g16 (8 tokens) of feature row f in a feature-major tile
+// Feature order inside LDS rows and registers.  A thread never holds eight consecutive
+// features: its 16 bytes are features {16G+4j .. +3} and {16G+8+4j .. +3} (G = 0..7,
+// j = 0..1), fetched as two 8-byte loads.  Token-major rows store these 16-byte units at
+// index 2G+j, so that lane half hh of an MFMA operand, reading unit 2k+hh, receives
+// features {16k+4hh .. +3, 16k+8+4hh .. +3}: exactly the rows 8g+4hh+r (g = 2u, 2u+1)
+// that the same lane holds of a 32x32 accumulator tile.  Accumulators can therefore be
+// multiplied against LDS rows with single 16-byte reads, and one set of X fragments
+// serves both the score product and the state product.
+struct LoaderRole {
+  int G, j;    // feature group and half handled by this thread
+  int rowq;    // X: row within a 16-row band; Y/Z: group of four rows
+};
+// X tile: 16 consecutive lanes fetch one 256-byte row
+__device__ __forceinline__ LoaderRole x_role(int tid) {
+  LoaderRole r;
+  r.G = (tid >> 1) & 7;
+  r.j = tid & 1;
+  r.rowq = tid >> 4;
+  return r;
+}
+// Y / Z tiles (also stored transposed): lane bits are dealt so that any 16 consecutive
+// lanes cover 8 feature units x 2 row groups -- 16 distinct 8-byte slots of the
+// feature-major tile, i.e. conflict-free ds_write_b64
+__device__ __forceinline__ LoaderRole yz_role(int tid) {
+  LoaderRole r;
+  r.j = tid & 1;
+  r.G = ((tid >> 1) & 3) | (((tid >> 4) & 1) << 2);
+  r.rowq = ((tid >> 3) & 1) | ((tid >> 5) << 1);
+  return r;
+}
+
+// byte offset of 16-byte granule g16 (8 tokens) of feature row f in a feature-major tile.
+// The XOR term varies with f bits 0-2 (consecutive rows read by consecutive lanes) and
+// with bits 2,4,5 (the rows written by 16 consecutive loader lanes).
 __device__ __forceinline__ int tr_off(int f, int g16) {
-  return f * LDT + (((g16 ^ f ^ (f >> 3)) & 7) << 4);
+  return f * LDT + (((g16 ^ (f & 7) ^ ((f >> 4) & 3)) & 7) << 4);
 }
 
 // l^x for x >= 0
@@ -84,16 +121,16 @@ __device__ __forceinline__ float decay(float s_log2e, float x) {
   return __builtin_amdgcn_exp2f(-s_log2e * x);
 }
 
-// Writes four rows (tokens 4*rowgrp .. +3) x eight features (8*dchunk .. +7) into a
+// Writes four rows (tokens 4*rowq .. +3) x the thread's eight features into a
 // feature-major tile: eight 8-byte stores, one per feature, each holding the four
 // tokens; `w[r]` scales token r before rounding (SCALE), else bits are moved as is.
 template <bool SCALE>
-__device__ __forceinline__ void store_transposed(char *tile, const uint4 (&rows)[4], int dchunk,
-                                                 int rowgrp, const float (&w)[4]) {
+__device__ __forceinline__ void store_transposed(char *tile, const u32x4 (&rows)[4],
+                                                 const LoaderRole &role, const float (&w)[4]) {
 #pragma unroll
   for (int x = 0; x < 8; ++x) {
-    const int f = 8 * dchunk + x;
-    uint2 out;
+    const int f = 16 * role.G + 8 * (x >> 2) + 4 * role.j + (x & 3);
+    u32x2 out;
     if (SCALE) {
       out.x = pack_bf16(bf_elem(rows[0], x) * w[0], bf_elem(rows[1], x) * w[1]);
       out.y = pack_bf16(bf_elem(rows[2], x) * w[2], bf_elem(rows[3], x) * w[3]);
@@ -101,8 +138,20 @@ __device__ __forceinline__ void store_transposed(char *tile, const uint4 (&rows)
       out.x = bf_bits(rows[0], x) | (bf_bits(rows[1], x) << 16);
       out.y = bf_bits(rows[2], x) | (bf_bits(rows[3], x) << 16);
     }
-    *reinterpret_cast<uint2 *>(tile + tr_off(f, rowgrp >> 1) + ((rowgrp & 1) << 3)) = out;
+    *reinterpret_cast<u32x2 *>(tile + tr_off(f, role.rowq >> 1) + ((role.rowq & 1) << 3)) = out;
   }
+}
+
+// the thread's two 8-byte pieces of one 128-feature row (pointer to the row start)
+__device__ __forceinline__ u32x4 load_row_pieces(const u32x2 *row, const LoaderRole &role) {
+  const u32x2 lo = row[4 * role.G + role.j];
+  const u32x2 hi = row[4 * role.G + 2 + role.j];
+  u32x4 r;
+  r.x = lo.x;
+  r.y = lo.y;
+  r.z = hi.x;
+  r.w = hi.y;
+  return r;
 }
 
 struct SegWork {
@@ -110,10 +159,11 @@ struct SegWork {
   int64_t tok0;  // first token of the segment
   int nblk;      // 64-token blocks in it
 };
-__device__ __forceinline__ SegWork seg_work(const Geom &g) {
+// `item` enumerates (b*h, segment) pairs
+__device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
   SegWork r;
-  r.bh = blockIdx.x / g.n_seg;
-  r.seg = blockIdx.x - r.bh * g.n_seg;
+  r.bh = item / g.n_seg;
+  r.seg = item - r.bh * g.n_seg;
   r.tok0 = (int64_t)r.seg * g.seg_len;
   int64_t t1 = r.tok0 + g.seg_len;
   if (t1 > g.n) t1 = g.n;
@@ -123,23 +173,23 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g) {
 
 // ------------------------------------------------------------------------------
 template <bool REV, bool TRANS>
-__global__ void __launch_bounds__(NTHR, 2)
-la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
-         const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
-         Geom g) {
-  extern __shared__ __align__(16) char smem[];
+__device__ __forceinline__ void
+apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
+           const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
+           const Geom &g, int item, char *smem) {
   const int tid = threadIdx.x;
   const int lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
-  const int chunk = tid & 15, rowq = tid >> 4;  // loader roles: 16-byte column, row / row group
+  const LoaderRole xr = x_role(tid), yr = yz_role(tid);
+  const int chunk = tid & 15, rowq = tid >> 4;  // output copy role: 16-byte column, row
 
-  const SegWork sw = seg_work(g);
+  const SegWork sw = seg_work(g, item);
   const float sl = S[sw.bh % g.h] * LOG2E;
   const int64_t base = ((int64_t)sw.bh * g.n + sw.tok0) * F;
-  const uint4 *Xg = reinterpret_cast<const uint4 *>(X + base);
-  const uint4 *Yg = reinterpret_cast<const uint4 *>(Y + base);
-  const uint4 *Zg = reinterpret_cast<const uint4 *>(Z + base);
-  uint4 *Og = reinterpret_cast<uint4 *>(Out + base);
+  const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + base);
+  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + base);
+  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + base);
+  u32x4 *Og = reinterpret_cast<u32x4 *>(Out + base);
 
   // ---- constants (all exponents <= 0)
   const float blockdec = decay(sl, (float)BLK);
@@ -152,7 +202,7 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
   float kdec[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int b = 4 * rowq + r;
+    const int b = 4 * yr.rowq + r;
     kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
   }
   const int qI = w >> 1, qJ = w & 1;  // score quadrant of this wave: queries 32*qI.., keys 32*qJ..
@@ -178,26 +228,26 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
   }
 
   // ---- block loader: registers <- global, LDS <- registers
-  uint4 nx[4], ny[4], nz[4];
-  auto issue_loads = [&](int blk) {
-    const int64_t off = (int64_t)blk * (BLK * F / 8);  // in 16-byte units
+  u32x4 nx[4], ny[4], nz[4];
+  auto issue_loads = [&](int blk) __attribute__((always_inline)) {
+    const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units (32 per row)
 #pragma unroll
-    for (int it = 0; it < 4; ++it) nx[it] = Xg[off + (rowq + 16 * it) * 16 + chunk];
+    for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      ny[r] = Yg[off + (4 * rowq + r) * 16 + chunk];
-      nz[r] = Zg[off + (4 * rowq + r) * 16 + chunk];
+      ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
+      nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
     }
   };
-  auto fill_lds = [&]() {
+  auto fill_lds = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < 4; ++it)
-      *reinterpret_cast<uint4 *>(smem + OFF_XN + (rowq + 16 * it) * LDN + chunk * 16) = nx[it];
+      *reinterpret_cast<u32x4 *>(smem + OFF_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      *reinterpret_cast<uint4 *>(smem + OFF_YN + (4 * rowq + r) * LDN + chunk * 16) = ny[r];
-    store_transposed<true>(smem + OFF_YT, ny, chunk, rowq, kdec);
-    store_transposed<false>(smem + OFF_ZT, nz, chunk, rowq, kdec);
+      *reinterpret_cast<u32x4 *>(smem + OFF_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
+    store_transposed<true>(smem + OFF_YT, ny, yr, kdec);
+    store_transposed<false>(smem + OFF_ZT, nz, yr, kdec);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
@@ -210,16 +260,37 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
 
-    // (1) score quadrant, transposed: sc[4g+r] = y_b . x_a, b = 32qJ+8g+4hh+r, a = 32qI+c
-    if (q_active) {
-      floatx16 sc;
+    // (1) one sweep over the 8 feature steps feeds two products from the same X fragments:
+    //     state term, transposed:  acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
+    //     score quadrant, transposed: sc[4g+r] = y_b . x_a, b = 32qJ+8g+4hh+r, a = 32qI+c
+    floatx16 acc[2], sc;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+    for (int r = 0; r < 16; ++r) {
+      acc[0][r] = 0.f;
+      acc[1][r] = 0.f;
+      sc[r] = 0.f;
+    }
+    {
+      const char *x0 = smem + OFF_XN + c * LDN + hh * 16;
+      const char *x1 = x0 + 32 * LDN;
       const char *ya = smem + OFF_YN + (32 * qJ + c) * LDN + hh * 16;
-      const char *xb = smem + OFF_XN + (32 * qI + c) * LDN + hh * 16;
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds16(ya + u * 32), lds16(xb + u * 32), sc, 0, 0, 0);
+      for (int ks = 0; ks < 8; ++ks) {
+        const int T = ks >> 1, u = ks & 1;
+        Frag a;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) a.w[p] = pack_bf16(st[T][8 * u + 2 * p], st[T][8 * u + 2 * p + 1]);
+        const bf16x8 xf0 = lds16(x0 + ks * 32);
+        const bf16x8 xf1 = lds16(x1 + ks * 32);
+        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, xf0, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, xf1, acc[1], 0, 0, 0);
+        if (q_active) {
+          const bf16x8 yf = lds16(ya + ks * 32);
+          sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yf, qI ? xf1 : xf0, sc, 0, 0, 0);
+        }
+      }
+    }
+    if (q_active) {
       const int a = 32 * qI + c;
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
@@ -230,35 +301,12 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
           const int dist = REV ? b - a : a - b;
           m[r] = dist >= 0 ? sc[4 * gq + r] * decay(sl, (float)dist) : 0.f;
         }
-        uint2 o;
+        u32x2 o;
         o.x = pack_bf16(m[0], m[1]);
         o.y = pack_bf16(m[2], m[3]);
-        *reinterpret_cast<uint2 *>(smem + OFF_SC + a * LDSC + (32 * qJ + 8 * gq + 4 * hh) * 2) = o;
+        *reinterpret_cast<u32x2 *>(smem + OFF_SC + a * LDSC + (32 * qJ + 8 * gq + 4 * hh) * 2) = o;
       }
     }
-
-    // (2) state term, transposed: acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
-    floatx16 acc[2];
-#pragma unroll
-    for (int I = 0; I < 2; ++I)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[I][r] = 0.f;
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        Frag a;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) a.w[p] = pack_bf16(st[T][8 * u + 2 * p], st[T][8 * u + 2 * p + 1]);
-#pragma unroll
-        for (int I = 0; I < 2; ++I) {
-          const char *xp = smem + OFF_XN + (32 * I + c) * LDN + (32 * T + 16 * u + 4 * hh) * 2;
-          Frag b;
-          b.h[0] = *reinterpret_cast<const uint2 *>(xp);
-          b.h[1] = *reinterpret_cast<const uint2 *>(xp + 16);
-          acc[I] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, acc[I], 0, 0, 0);
-        }
-      }
 #pragma unroll
     for (int I = 0; I < 2; ++I)
 #pragma unroll
@@ -297,10 +345,10 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
     for (int I = 0; I < 2; ++I)
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
-        uint2 o;
+        u32x2 o;
         o.x = pack_bf16(acc[I][4 * gq + 0], acc[I][4 * gq + 1]);
         o.y = pack_bf16(acc[I][4 * gq + 2], acc[I][4 * gq + 3]);
-        *reinterpret_cast<uint2 *>(smem + OFF_YN + (32 * I + c) * LDN + (32 * w + 8 * gq + 4 * hh) * 2) = o;
+        *reinterpret_cast<u32x2 *>(smem + OFF_YN + (32 * I + c) * LDN + (32 * w + 8 * gq + 4 * hh) * 2) = o;
       }
     __syncthreads();  // B: staged output complete; YT / ZT / score no longer read
     {
@@ -308,7 +356,8 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int row = rowq + 16 * r4;
-        Og[off + row * 16 + chunk] = *reinterpret_cast<const uint4 *>(smem + OFF_YN + row * LDN + chunk * 16);
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(smem + OFF_YN + row * LDN + chunk * 16),
+                                    &Og[off + row * 16 + chunk]);
       }
     }
     if (more) {
@@ -317,6 +366,41 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
       __syncthreads();  // D: next block visible
     }
   }
+}
+
+// Work items are taken in descending order: the pre-pass that ran just before this
+// kernel read the tensors front to back, so the tail is what the memory-side cache
+// still holds.
+template <bool REV, bool TRANS>
+__global__ void __launch_bounds__(NTHR, 2)
+la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
+         const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
+         Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  apply_body<REV, TRANS>(X, Y, Z, S, states, Out, g, (int)(gridDim.x - 1 - blockIdx.x), smem);
+}
+
+// The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
+// work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
+// the triple is spread over block indices 8 apart so that all three land on the same
+// XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
+__global__ void __launch_bounds__(NTHR, 2)
+la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
+        const bf16_t *__restrict__ DO, const float *__restrict__ S,
+        const float *__restrict__ kv_states, const float *__restrict__ dkv_states,
+        bf16_t *__restrict__ DQ, bf16_t *__restrict__ DK, bf16_t *__restrict__ DV, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  const int n_items = g.b * g.h * g.n_seg;
+  const int grp = blockIdx.x / 24, r = blockIdx.x - grp * 24;
+  const int role = r >> 3;
+  const int item = n_items - 1 - (grp * 8 + (r & 7));
+  if (item < 0) return;
+  if (role == 0)
+    apply_body<false, true>(DO, V, K, S, kv_states, DQ, g, item, smem);
+  else if (role == 1)
+    apply_body<true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem);
+  else
+    apply_body<true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem);
 }
 
 // ------------------------------------------------------------------------------
@@ -330,19 +414,19 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
   const int tid = threadIdx.x;
   const int lane = tid & 63, w = tid >> 6;
   const int c = lane & 31, hh = lane >> 5;
-  const int chunk = tid & 15, rowq = tid >> 4;
+  const LoaderRole yr = yz_role(tid);
 
-  const SegWork sw = seg_work(g);
+  const SegWork sw = seg_work(g, (int)blockIdx.x);
   const float sl = S[sw.bh % g.h] * LOG2E;
   const int64_t base = ((int64_t)sw.bh * g.n + sw.tok0) * F;
-  const uint4 *Yg = reinterpret_cast<const uint4 *>(Y + base);
-  const uint4 *Zg = reinterpret_cast<const uint4 *>(Z + base);
+  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + base);
+  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + base);
 
   const float blockdec = decay(sl, (float)BLK);
   float kdec[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int b = 4 * rowq + r;
+    const int b = 4 * yr.rowq + r;
     kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
   }
 
@@ -352,18 +436,18 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
 
-  uint4 ny[4], nz[4];
-  auto issue_loads = [&](int blk) {
-    const int64_t off = (int64_t)blk * (BLK * F / 8);
+  u32x4 ny[4], nz[4];
+  auto issue_loads = [&](int blk) __attribute__((always_inline)) {
+    const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      ny[r] = Yg[off + (4 * rowq + r) * 16 + chunk];
-      nz[r] = Zg[off + (4 * rowq + r) * 16 + chunk];
+      ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
+      nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
     }
   };
-  auto fill_lds = [&](int buf) {
-    store_transposed<true>(smem[buf], ny, chunk, rowq, kdec);
-    store_transposed<false>(smem[buf] + F * LDT, nz, chunk, rowq, kdec);
+  auto fill_lds = [&](int buf) __attribute__((always_inline)) {
+    store_transposed<true>(smem[buf], ny, yr, kdec);
+    store_transposed<false>(smem[buf] + F * LDT, nz, yr, kdec);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
@@ -400,10 +484,21 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
       sp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
 }
 
+// Dynamic LDS above the default limit has to be granted once per kernel and device.
 template <class K>
 int raise_lds(K kernel) {
-  return (int)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  APPLY_LDS);
+  static thread_local const void *granted_fn = nullptr;
+  static thread_local int granted_dev = -1;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (granted_fn == (const void *)kernel && granted_dev == dev) return 0;
+  e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, APPLY_LDS);
+  if (e == hipSuccess) {
+    granted_fn = (const void *)kernel;
+    granted_dev = dev;
+  }
+  return (int)e;
 }
 
 template <bool REV, bool TRANS>
@@ -415,6 +510,19 @@ int launch_apply(const void *x, const void *y, const void *z, const float *s, co
   ProfScope prof(KC_APPLY, st);
   la_apply<REV, TRANS><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
                                                       (const bf16_t *)z, s, states, (bf16_t *)out, g);
+  return (int)hipGetLastError();
+}
+
+int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
+                hipStream_t st) {
+  int rc = raise_lds(la_bwd3);
+  if (rc) return rc;
+  const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
+  const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
+  ProfScope prof(KC_BWD3, st);
+  la_bwd3<<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k, (const bf16_t *)a.v,
+                                         (const bf16_t *)a.d_o, a.s, kv_states, dkv_states,
+                                         (bf16_t *)a.dq, (bf16_t *)a.dk, (bf16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
@@ -453,9 +561,7 @@ int mfma_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  if ((rc = launch_apply<false, true>(a.d_o, a.v, a.k, a.s, kv_states, a.dq, g, st))) return rc;
-  if ((rc = launch_apply<true, false>(a.k, a.q, a.d_o, a.s, dkv_states, a.dv, g, st))) return rc;
-  return launch_apply<true, true>(a.v, a.d_o, a.q, a.s, dkv_states, a.dk, g, st);
+  return launch_bwd3(a, kv_states, dkv_states, g, st);
 }
 
 }  // namespace lasp
