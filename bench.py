@@ -31,7 +31,11 @@ FLOP_FWD_PER_TH = 98304        # 2Bd + 2Be + 4de at B=64, d=e=128
 FLOP_BWD_PER_TH = 245760       # 6Bd + 4Be + 10de
 BYTES_FWD_PER_TH = 1024        # read Q,K,V + write O, bf16
 BYTES_BWD_PER_TH = 1792        # read Q,K,V,dO + write dQ,dK,dV
-APPLY_LAUNCHES_PER_STEP = 4    # O, dQ, dV, dK
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
+# (profiles/pmc_hbm_bytes_config2.txt); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0, the
+# factors a plain 1 GiB device copy shows for the same counters.
+TRAFFIC_BWD3_BYTES = None
+TRAFFIC_APPLY_BYTES = None
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
@@ -141,12 +145,18 @@ def main():
     for _ in range(args.steps):
         step()
     prof = _abi.profile_end()
-    apply_ms, apply_n = prof["apply"]
-    apply_avg_ms = apply_ms / max(apply_n, 1)
-
     th = B * H * N
-    alg_bytes_per_launch = (BYTES_FWD_PER_TH + BYTES_BWD_PER_TH) * th / APPLY_LAUNCHES_PER_STEP
-    achieved = alg_bytes_per_launch / (apply_avg_ms * 1e-3) / 1e9
+
+    def roof(kernel, cls, alg_bytes, traffic):
+        ms, cnt = prof[cls]
+        avg_ms = ms / max(cnt, 1)
+        achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+        return {
+            "kernel": kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+            "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": avg_ms, "launches": cnt,
+        }
+
     flop_step = (FLOP_FWD_PER_TH + FLOP_BWD_PER_TH) * th
     tflops = flop_step / (ms_step * 1e-3) / 1e12
 
@@ -175,18 +185,10 @@ def main():
         "frac_bf16_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS,
         "step_algorithmic_gbs": (BYTES_FWD_PER_TH + BYTES_BWD_PER_TH) * th / (ms_step * 1e-3) / 1e9,
         "kernel_ms": {name: {"total_ms": ms, "launches": cnt} for name, (ms, cnt) in prof.items() if cnt},
-        "roofline": {
-            "kernel": "la_apply",
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
-            "algorithmic_bytes_per_launch": alg_bytes_per_launch,
-            "avg_launch_ms": apply_avg_ms,
-            "launches": apply_n,
-        },
+        # dominant kernel: la_bwd3 (one launch = the whole backward sweep: reads Q,K,V,dO, writes dQ,dK,dV)
+        "roofline": roof("la_bwd3", "bwd3", BYTES_BWD_PER_TH * th, TRAFFIC_BWD3_BYTES),
+        # second kernel: la_apply (one launch = the forward sweep: reads Q,K,V, writes O)
+        "roofline_fwd": roof("la_apply", "apply", BYTES_FWD_PER_TH * th, TRAFFIC_APPLY_BYTES),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
