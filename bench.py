@@ -34,8 +34,8 @@ BYTES_BWD_PER_TH = 1792        # read Q,K,V,dO + write dQ,dK,dV
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
 # (profiles/pmc_hbm_bytes_config2.txt); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0, the
 # factors a plain 1 GiB device copy shows for the same counters.
-TRAFFIC_BWD3_BYTES = None
-TRAFFIC_APPLY_BYTES = None
+TRAFFIC_BWD3_BYTES = 2824264 * 1024   # 2 x 1 018 916 KiB fetched + 786 432 KiB written
+TRAFFIC_APPLY_BYTES = 1081505 * 1024  # 2 x 409 681 KiB fetched + 262 144 KiB written
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
@@ -82,7 +82,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprofv3 byte counters)")

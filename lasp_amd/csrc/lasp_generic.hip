@@ -333,17 +333,25 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   const float full = expf(-s * (float)g.seg_len);
   const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
   const float tail = expf(-s * (float)last_len);
-  if (!reverse) {
-    for (int sg = 0; sg < g.n_seg; ++sg) {
-      const float local = p[(int64_t)sg * de];
-      p[(int64_t)sg * de] = run;
-      run = fmaf(sg == g.n_seg - 1 ? tail : full, run, local);
+  // The loads do not depend on the recurrence: fetch a batch of segment states, then run
+  // the serial chain over the batch (forward: segments ascending; reverse: descending).
+  constexpr int BATCH = 8;
+  for (int done = 0; done < g.n_seg; done += BATCH) {
+    float local[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int k = done + u;
+      const int sg = reverse ? g.n_seg - 1 - k : k;
+      local[u] = k < g.n_seg ? p[(int64_t)sg * de] : 0.f;
     }
-  } else {
-    for (int sg = g.n_seg - 1; sg >= 0; --sg) {
-      const float local = p[(int64_t)sg * de];
-      p[(int64_t)sg * de] = run;
-      run = fmaf(sg == g.n_seg - 1 ? tail : full, run, local);
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) {
+      const int k = done + u;
+      if (k < g.n_seg) {
+        const int sg = reverse ? g.n_seg - 1 - k : k;
+        p[(int64_t)sg * de] = run;
+        run = fmaf(sg == g.n_seg - 1 ? tail : full, run, local[u]);
+      }
     }
   }
   if (carry_out) carry_out[idx] = run;

@@ -368,16 +368,13 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
   }
 }
 
-// Work items are taken in descending order: the pre-pass that ran just before this
-// kernel read the tensors front to back, so the tail is what the memory-side cache
-// still holds.
 template <bool REV, bool TRANS>
 __global__ void __launch_bounds__(NTHR, 2)
 la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
          const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
          Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<REV, TRANS>(X, Y, Z, S, states, Out, g, (int)(gridDim.x - 1 - blockIdx.x), smem);
+  apply_body<REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
@@ -409,7 +406,7 @@ la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t
 template <bool REV>
 __global__ void __launch_bounds__(NTHR, 2)
 la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const float *__restrict__ S,
-             float *__restrict__ states, Geom g) {
+             float *__restrict__ states, Geom g, int skip_seg) {
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
   const int tid = threadIdx.x;
   const int lane = tid & 63, w = tid >> 6;
@@ -417,6 +414,7 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
   const LoaderRole yr = yz_role(tid);
 
   const SegWork sw = seg_work(g, (int)blockIdx.x);
+  if (sw.seg == skip_seg) return;  // the scan's final segment feeds only the outgoing carry
   const float sl = S[sw.bh % g.h] * LOG2E;
   const int64_t base = ((int64_t)sw.bh * g.n + sw.tok0) * F;
   const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + base);
@@ -526,12 +524,15 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
+// carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
+// segment it visits last (whose own state feeds nothing else) is skipped.
 template <bool REV>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
-                 hipStream_t st) {
+                 bool carry_wanted, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g);
+  la_seg_state<REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g, skip_seg);
   return (int)hipGetLastError();
 }
 
@@ -541,7 +542,7 @@ int mfma_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.seg_states, g, st))) return rc;
+    if ((rc = launch_state<false>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
   return launch_apply<false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
@@ -551,13 +552,13 @@ int mfma_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.ws_kv, g, st))) return rc;
+    if ((rc = launch_state<false>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<true>(a.q, a.d_o, a.s, a.ws_dkv, g, st))) return rc;
+    if ((rc = launch_state<true>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
