@@ -311,17 +311,23 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
     for (int I = 0; I < 2; ++I)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[I][r] *= qdec[I];
+    // the state has been consumed by the sweep: decay it now, ahead of the update in (4)
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
 
     __syncthreads();  // A: score tile complete; XN / YN no longer read
 
     // (3) intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
+    //     (token step outermost, so that consecutive MFMAs write different accumulators)
     bf16x8 zf[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
 #pragma unroll
-    for (int I = 0; I < 2; ++I)
+    for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int I = 0; I < 2; ++I) {
         const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
         if (needed) {
           const bf16x8 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
@@ -329,16 +335,13 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
         }
       }
 
-    // (4) state update: St <- l^64 St + (scaled Y)^T Z
+    // (4) state update: St <- l^64 St + (scaled Y)^T Z   (the decay was applied after the sweep)
 #pragma unroll
-    for (int T = 0; T < 4; ++T) {
+    for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int T = 0; T < 4; ++T)
         st[T] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
             lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T], 0, 0, 0);
-    }
 
     // (5) stage the output tile (token-major, in the YN region) for coalesced stores
 #pragma unroll

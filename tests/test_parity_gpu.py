@@ -111,6 +111,8 @@ def test_argument_errors(gpu_device):
 @pytest.mark.parametrize("state", [False, True])
 @pytest.mark.parametrize("b,h,n,seg", [
     (1, 1, 64, 0), (1, 2, 128, 64), (1, 2, 256, 0), (2, 3, 512, 128), (1, 4, 1024, 256), (1, 2, 2048, 2048),
+    (2, 2, 320, 256),   # last segment shorter than the others
+    (3, 5, 192, 128),   # b*h*n_seg not a multiple of 8 (partial group of backward workgroup triples)
 ])
 def test_mfma_bf16(gpu_device, b, h, n, seg, state):
     from lasp_amd import _abi
