@@ -152,7 +152,7 @@ def _slopes(s: torch.Tensor, h: int, dev) -> torch.Tensor:
     return s.detach().to(device=dev, dtype=torch.float32).contiguous()
 
 
-def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
+def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     """Enqueues the forward of one chunk.  Returns (o, seg_states, seg_len).
 
     seg_states is the (b, h, n_seg, d, e) float32 array of states entering each
@@ -180,7 +180,7 @@ def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     return o, states, seg_len
 
 
-def chunk_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):
+def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):
     """Enqueues the backward of one chunk.  Returns (dq, dk, dv)."""
     lib = load()
     dev = _check_dev(q, k, v, do, kv_in, dkv_in, dkv_out, kv_seg_states)
@@ -211,3 +211,62 @@ def chunk_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_stat
     if rc:
         _raise(rc, "lasp_chunk_bwd")
     return dq, dk, dv
+
+
+# ---------------------------------------------------------------------------------------
+# Narrow heads on the MFMA kernels.  The bf16 MFMA kernels take d = e = 128 only.  A bf16
+# call with narrower features (the reference's own test uses e = 64, tests/test.py:95) is
+# zero-padded to 128 here: zero feature columns add nothing to q.k, to the outputs or to the
+# states, so the results are exact, and the call runs an order of magnitude faster than on
+# the generic fp32-FMA kernels.  Everything else goes to the library unchanged.
+_MFMA_F = 128
+
+
+def _pad_to_mfma(q, v) -> bool:
+    n, d, e = q.shape[2], q.shape[3], v.shape[3]
+    return q.dtype == torch.bfloat16 and n % 64 == 0 and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
+
+
+def _pad_last(t, size):
+    return t if t.shape[-1] == size else torch.nn.functional.pad(t, (0, size - t.shape[-1]))
+
+
+def _pad_state(t, d, e):
+    if t is None:
+        return None
+    out = torch.zeros(t.shape[0], t.shape[1], _MFMA_F, _MFMA_F, dtype=torch.float32, device=t.device)
+    out[:, :, :d, :e] = t
+    return out
+
+
+def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
+    """Forward of one chunk: (o, seg_states, seg_len).  See _chunk_fwd_exact; narrow bf16 heads are padded."""
+    if q.dim() != 4 or v.dim() != 4 or not _pad_to_mfma(q, v):
+        return _chunk_fwd_exact(q, k, v, s, kv_in, kv_out, seg_len)
+    b, h, n, d, e = _shapes(q, k, v)
+    _check_state("kv_in", kv_in, b, h, d, e)
+    _check_state("kv_out", kv_out, b, h, d, e)
+    kv_out_p = None if kv_out is None else torch.empty(b, h, _MFMA_F, _MFMA_F, dtype=torch.float32, device=q.device)
+    o, states, seg_len = _chunk_fwd_exact(_pad_last(q, _MFMA_F), _pad_last(k, _MFMA_F), _pad_last(v, _MFMA_F), s,
+                                          _pad_state(kv_in, d, e), kv_out_p, seg_len)
+    if kv_out is not None:
+        kv_out.copy_(kv_out_p[:, :, :d, :e])
+    return o[..., :e].contiguous(), states, seg_len
+
+
+def chunk_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):
+    """Backward of one chunk: (dq, dk, dv).  See _chunk_bwd_exact; narrow bf16 heads are padded
+    (kv_seg_states must then be what chunk_fwd returned for the same call)."""
+    if q.dim() != 4 or v.dim() != 4 or not _pad_to_mfma(q, v):
+        return _chunk_bwd_exact(q, k, v, s, do, kv_in, dkv_in, dkv_out, kv_seg_states, seg_len)
+    b, h, n, d, e = _shapes(q, k, v)
+    _check_state("kv_in", kv_in, b, h, d, e)
+    _check_state("dkv_in", dkv_in, b, h, d, e)
+    _check_state("dkv_out", dkv_out, b, h, d, e)
+    dkv_out_p = None if dkv_out is None else torch.empty(b, h, _MFMA_F, _MFMA_F, dtype=torch.float32, device=q.device)
+    dq, dk, dv = _chunk_bwd_exact(_pad_last(q, _MFMA_F), _pad_last(k, _MFMA_F), _pad_last(v, _MFMA_F), s,
+                                  _pad_last(do, _MFMA_F), _pad_state(kv_in, d, e), _pad_state(dkv_in, d, e),
+                                  dkv_out_p, kv_seg_states, seg_len)
+    if dkv_out is not None:
+        dkv_out.copy_(dkv_out_p[:, :, :d, :e])
+    return dq[..., :d].contiguous(), dk[..., :d].contiguous(), dv[..., :e].contiguous()

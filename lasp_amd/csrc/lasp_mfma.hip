@@ -270,6 +270,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
       acc[1][r] = 0.f;
       sc[r] = 0.f;
     }
+    __builtin_amdgcn_s_setprio(1);
     {
       const char *x0 = smem + OFF_XN + c * LDN + hh * 16;
       const char *x1 = x0 + 32 * LDN;
@@ -290,6 +291,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
         }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
     if (q_active) {
       const int a = 32 * qI + c;
 #pragma unroll
@@ -324,6 +326,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
     bf16x8 zf[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
@@ -343,6 +346,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
         st[T] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
             lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T], 0, 0, 0);
 
+    __builtin_amdgcn_s_setprio(0);
     // (5) stage the output tile (token-major, in the YN region) for coalesced stores
 #pragma unroll
     for (int I = 0; I < 2; ++I)

@@ -52,8 +52,8 @@ def test_generic_fp32_small(gpu_device, shape, state):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_generic_low_precision_io(gpu_device, dtype):
-    # e != d keeps these on the generic kernels (the reference test shape has e = 64)
-    inp = make_inputs(2, 12, 512, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    # ragged n keeps these on the generic kernels
+    inp = make_inputs(2, 12, 500, 128, 64, dtype, seed=3, state=True, state_std=1.0)
     s = O.slopes_alibi(12)
     got = run_abi(inp, s, gpu_device)
     check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
@@ -149,3 +149,14 @@ def test_mfma_cached_states_equal_recompute(gpu_device):
     c = run_abi(inp, s, gpu_device, seg_len=256, cache=True)
     for name in ("dq", "dk", "dv", "dkv_out"):
         assert torch.equal(a[name], c[name]), name
+
+
+@pytest.mark.parametrize("d,e", [(128, 64), (64, 128), (64, 64), (96, 32)])
+def test_narrow_bf16_heads_run_padded_on_mfma(gpu_device, d, e):
+    # the reference's own test shape has e = 64 (tests/test.py:95): zero-padded to 128, exact
+    inp = make_inputs(2, 3, 512, d, e, torch.bfloat16, seed=d + e, state=True, state_std=1.0)
+    s = O.slopes_alibi(3)
+    for cache in (False, True):
+        got = run_abi(inp, s, gpu_device, seg_len=128, cache=cache)
+        assert got["o"].shape[-1] == e and got["dq"].shape[-1] == d and got["kv_out"].shape[-2:] == (d, e)
+        check(got, oracle(inp, s), 2e-2, what=f"padded d={d} e={e} cache={cache}")
