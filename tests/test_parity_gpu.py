@@ -52,8 +52,8 @@ def test_generic_fp32_small(gpu_device, shape, state):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_generic_low_precision_io(gpu_device, dtype):
-    # ragged n keeps these on the generic kernels
-    inp = make_inputs(2, 12, 500, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    # n < 64 (bf16) and fp16 keep these on the generic kernels
+    inp = make_inputs(2, 12, 500 if dtype == torch.float16 else 50, 128, 64, dtype, seed=3, state=True, state_std=1.0)
     s = O.slopes_alibi(12)
     got = run_abi(inp, s, gpu_device)
     check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
@@ -160,3 +160,14 @@ def test_narrow_bf16_heads_run_padded_on_mfma(gpu_device, d, e):
         got = run_abi(inp, s, gpu_device, seg_len=128, cache=cache)
         assert got["o"].shape[-1] == e and got["dq"].shape[-1] == d and got["kv_out"].shape[-2:] == (d, e)
         check(got, oracle(inp, s), 2e-2, what=f"padded d={d} e={e} cache={cache}")
+
+
+@pytest.mark.parametrize("n,d,e", [(2047, 128, 128), (65, 128, 128), (700, 128, 64)])
+def test_ragged_bf16_length_is_split_head_mfma_tail_generic(gpu_device, n, d, e):
+    inp = make_inputs(1, 3, n, d, e, torch.bfloat16, seed=n, state=True, state_std=1.0)
+    s = O.slopes_alibi(3)
+    ref = oracle(inp, s)
+    for cache in (False, True):
+        got = run_abi(inp, s, gpu_device, cache=cache)
+        assert got["o"].shape == inp["v"].shape and got["dq"].shape == inp["q"].shape
+        check(got, ref, 2e-2, what=f"ragged n={n} d={d} e={e} cache={cache}")
