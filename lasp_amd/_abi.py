@@ -220,11 +220,12 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
 # states, so the results are exact, and the call runs an order of magnitude faster than on
 # the generic fp32-FMA kernels.  Everything else goes to the library unchanged.
 _MFMA_F = 128
+_MFMA_DTYPES = (torch.bfloat16, torch.float16)
 
 
 def _pad_to_mfma(q, v) -> bool:
     n, d, e = q.shape[2], q.shape[3], v.shape[3]
-    return q.dtype == torch.bfloat16 and n % 64 == 0 and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
+    return q.dtype in _MFMA_DTYPES and n % 64 == 0 and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
 
 
 def _pad_last(t, size):
@@ -241,7 +242,7 @@ def _pad_state(t, d, e):
 
 def _ragged_for_mfma(q, v) -> bool:
     n, d, e = q.shape[2], q.shape[3], v.shape[3]
-    return q.dtype == torch.bfloat16 and n % 64 != 0 and n > 64 and d <= _MFMA_F and e <= _MFMA_F
+    return q.dtype in _MFMA_DTYPES and n % 64 != 0 and n > 64 and d <= _MFMA_F and e <= _MFMA_F
 
 
 # A bf16 chunk whose length is not a multiple of 64 is cut at the last multiple: the head runs

@@ -93,7 +93,7 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
 }
 
 bool mfma_eligible(const Geom &g, int dtype) {
-  return dtype == LASP_DTYPE_BF16 && g.d == 128 && g.e == 128 && g.n % 64 == 0;
+  return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && g.d == 128 && g.e == 128 && g.n % 64 == 0;
 }
 
 size_t state_bytes_of(const Geom &g) {
@@ -199,7 +199,7 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
   }
   FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype) ? mfma_fwd(a, g, st) : generic_fwd(a, g, dtype, st);
+  rc = mfma_eligible(g, dtype) ? mfma_fwd(a, g, dtype, st) : generic_fwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_fwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }
@@ -236,7 +236,7 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
   }
   if (need_kv) a.ws_kv = wp;
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype) ? mfma_bwd(a, g, st) : generic_bwd(a, g, dtype, st);
+  rc = mfma_eligible(g, dtype) ? mfma_bwd(a, g, dtype, st) : generic_bwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_bwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }

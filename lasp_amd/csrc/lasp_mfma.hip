@@ -1,4 +1,4 @@
-// bf16 MFMA kernels for d = e = 128, n % 64 == 0 (gfx950, wave64).
+// bf16 / fp16 MFMA kernels for d = e = 128, n % 64 == 0 (gfx950, wave64).
 //
 // One kernel, `la_apply`, evaluates a causal (or anti-causal) decayed linear
 // attention over a segment of 64-token blocks given the state entering it:
@@ -31,6 +31,10 @@
 namespace lasp {
 namespace {
 
+// native vector types (HIP's uint4 / uint2 structs copy through memcpy, which can pin
+// a register array to scratch memory)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
@@ -54,24 +58,48 @@ constexpr int OFF_SC = OFF_ZT + F * LDT;
 constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
 constexpr float LOG2E = 1.4426950408889634f;
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  float2_t v = {lo, hi};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
-}
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
 
-union Frag {
-  bf16x8 v;
-  u32x4 q;
-  u32x2 h[2];
-  uint32_t w[4];
+// Element policies: the kernels move 16-bit elements as raw bits and only touch their value
+// in three places -- widening one element, rounding two floats into a packed pair, and the
+// MFMA itself.
+struct ElemBF16 {
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    float2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+  }
+  // `bits` holds the element in its low (odd = false) or high (odd = true) half
+  static __device__ __forceinline__ float widen(uint32_t word, bool odd) {
+    return __uint_as_float(odd ? (word & 0xffff0000u) : (word << 16));
+  }
+  static __device__ __forceinline__ floatx16 mfma(u32x4 a, u32x4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                   c, 0, 0, 0);
+  }
+};
+struct ElemF16 {
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    float2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
+  }
+  static __device__ __forceinline__ float widen(uint32_t word, bool odd) {
+    const f16x2_t h = __builtin_bit_cast(f16x2_t, word);
+    return (float)(odd ? h.y : h.x);
+  }
+  static __device__ __forceinline__ floatx16 mfma(u32x4 a, u32x4 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
+  }
 };
 
-__device__ __forceinline__ bf16x8 lds16(const char *p) { return *reinterpret_cast<const bf16x8 *>(p); }
+__device__ __forceinline__ u32x4 lds16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
-// element x (0..7) of a 16-byte group of bf16, widened to fp32
-__device__ __forceinline__ float bf_elem(const u32x4 &q, int x) {
+// element x (0..7) of a 16-byte group of 16-bit elements, widened to fp32
+template <class E>
+__device__ __forceinline__ float elem_f32(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
-  return __uint_as_float((x & 1) ? (w & 0xffff0000u) : (w << 16));
+  return E::widen(w, x & 1);
 }
 __device__ __forceinline__ uint32_t bf_bits(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
@@ -124,7 +152,7 @@ __device__ __forceinline__ float decay(float s_log2e, float x) {
 // Writes four rows (tokens 4*rowq .. +3) x the thread's eight features into a
 // feature-major tile: eight 8-byte stores, one per feature, each holding the four
 // tokens; `w[r]` scales token r before rounding (SCALE), else bits are moved as is.
-template <bool SCALE>
+template <class E, bool SCALE>
 __device__ __forceinline__ void store_transposed(char *tile, const u32x4 (&rows)[4],
                                                  const LoaderRole &role, const float (&w)[4]) {
 #pragma unroll
@@ -132,8 +160,8 @@ __device__ __forceinline__ void store_transposed(char *tile, const u32x4 (&rows)
     const int f = 16 * role.G + 8 * (x >> 2) + 4 * role.j + (x & 3);
     u32x2 out;
     if (SCALE) {
-      out.x = pack_bf16(bf_elem(rows[0], x) * w[0], bf_elem(rows[1], x) * w[1]);
-      out.y = pack_bf16(bf_elem(rows[2], x) * w[2], bf_elem(rows[3], x) * w[3]);
+      out.x = E::pack(elem_f32<E>(rows[0], x) * w[0], elem_f32<E>(rows[1], x) * w[1]);
+      out.y = E::pack(elem_f32<E>(rows[2], x) * w[2], elem_f32<E>(rows[3], x) * w[3]);
     } else {
       out.x = bf_bits(rows[0], x) | (bf_bits(rows[1], x) << 16);
       out.y = bf_bits(rows[2], x) | (bf_bits(rows[3], x) << 16);
@@ -172,7 +200,7 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 }
 
 // ------------------------------------------------------------------------------
-template <bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS>
 __device__ __forceinline__ void
 apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
@@ -246,8 +274,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       *reinterpret_cast<u32x4 *>(smem + OFF_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
-    store_transposed<true>(smem + OFF_YT, ny, yr, kdec);
-    store_transposed<false>(smem + OFF_ZT, nz, yr, kdec);
+    store_transposed<E, true>(smem + OFF_YT, ny, yr, kdec);
+    store_transposed<E, false>(smem + OFF_ZT, nz, yr, kdec);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
@@ -278,16 +306,18 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
         const int T = ks >> 1, u = ks & 1;
-        Frag a;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) a.w[p] = pack_bf16(st[T][8 * u + 2 * p], st[T][8 * u + 2 * p + 1]);
-        const bf16x8 xf0 = lds16(x0 + ks * 32);
-        const bf16x8 xf1 = lds16(x1 + ks * 32);
-        acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, xf0, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, xf1, acc[1], 0, 0, 0);
+        u32x4 a;
+        a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
+        a.y = E::pack(st[T][8 * u + 2], st[T][8 * u + 3]);
+        a.z = E::pack(st[T][8 * u + 4], st[T][8 * u + 5]);
+        a.w = E::pack(st[T][8 * u + 6], st[T][8 * u + 7]);
+        const u32x4 xf0 = lds16(x0 + ks * 32);
+        const u32x4 xf1 = lds16(x1 + ks * 32);
+        acc[0] = E::mfma(a, xf0, acc[0]);
+        acc[1] = E::mfma(a, xf1, acc[1]);
         if (q_active) {
-          const bf16x8 yf = lds16(ya + ks * 32);
-          sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(yf, qI ? xf1 : xf0, sc, 0, 0, 0);
+          const u32x4 yf = lds16(ya + ks * 32);
+          sc = E::mfma(yf, qI ? xf1 : xf0, sc);
         }
       }
     }
@@ -304,8 +334,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
           m[r] = dist >= 0 ? sc[4 * gq + r] * decay(sl, (float)dist) : 0.f;
         }
         u32x2 o;
-        o.x = pack_bf16(m[0], m[1]);
-        o.y = pack_bf16(m[2], m[3]);
+        o.x = E::pack(m[0], m[1]);
+        o.y = E::pack(m[2], m[3]);
         *reinterpret_cast<u32x2 *>(smem + OFF_SC + a * LDSC + (32 * qJ + 8 * gq + 4 * hh) * 2) = o;
       }
     }
@@ -323,7 +353,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 
     // (3) intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
     //     (token step outermost, so that consecutive MFMAs write different accumulators)
-    bf16x8 zf[4];
+    u32x4 zf[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
     __builtin_amdgcn_s_setprio(1);
@@ -333,8 +363,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
       for (int I = 0; I < 2; ++I) {
         const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
         if (needed) {
-          const bf16x8 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
-          acc[I] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(zf[u], b, acc[I], 0, 0, 0);
+          const u32x4 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
+          acc[I] = E::mfma(zf[u], b, acc[I]);
         }
       }
 
@@ -343,8 +373,7 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
     for (int u = 0; u < 4; ++u)
 #pragma unroll
       for (int T = 0; T < 4; ++T)
-        st[T] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-            lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T], 0, 0, 0);
+        st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
 
     __builtin_amdgcn_s_setprio(0);
     // (5) stage the output tile (token-major, in the YN region) for coalesced stores
@@ -353,8 +382,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         u32x2 o;
-        o.x = pack_bf16(acc[I][4 * gq + 0], acc[I][4 * gq + 1]);
-        o.y = pack_bf16(acc[I][4 * gq + 2], acc[I][4 * gq + 3]);
+        o.x = E::pack(acc[I][4 * gq + 0], acc[I][4 * gq + 1]);
+        o.y = E::pack(acc[I][4 * gq + 2], acc[I][4 * gq + 3]);
         *reinterpret_cast<u32x2 *>(smem + OFF_YN + (32 * I + c) * LDN + (32 * w + 8 * gq + 4 * hh) * 2) = o;
       }
     __syncthreads();  // B: staged output complete; YT / ZT / score no longer read
@@ -375,19 +404,20 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
   }
 }
 
-template <bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS>
 __global__ void __launch_bounds__(NTHR, 2)
 la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
          const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
          Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
+  apply_body<E, REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
 // work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
 // the triple is spread over block indices 8 apart so that all three land on the same
 // XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
+template <class E>
 __global__ void __launch_bounds__(NTHR, 2)
 la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
         const bf16_t *__restrict__ DO, const float *__restrict__ S,
@@ -400,17 +430,17 @@ la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    apply_body<false, true>(DO, V, K, S, kv_states, DQ, g, item, smem);
+    apply_body<E, false, true>(DO, V, K, S, kv_states, DQ, g, item, smem);
   else if (role == 1)
-    apply_body<true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem);
+    apply_body<E, true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem);
   else
-    apply_body<true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem);
+    apply_body<E, true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem);
 }
 
 // ------------------------------------------------------------------------------
 // A segment's own state:  causal  sum_b l^(L-b) y_b^T z_b ;  anti-causal  sum_b l^b y_b^T z_b
 // (b from the segment start, L its length), written token-free as 128 x 128 fp32.
-template <bool REV>
+template <class E, bool REV>
 __global__ void __launch_bounds__(NTHR, 2)
 la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
@@ -451,8 +481,8 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
     }
   };
   auto fill_lds = [&](int buf) __attribute__((always_inline)) {
-    store_transposed<true>(smem[buf], ny, yr, kdec);
-    store_transposed<false>(smem[buf] + F * LDT, nz, yr, kdec);
+    store_transposed<E, true>(smem[buf], ny, yr, kdec);
+    store_transposed<E, false>(smem[buf] + F * LDT, nz, yr, kdec);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
@@ -465,7 +495,7 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
     if (more) issue_loads(blk + step);
     const char *yt = smem[it & 1];
     const char *zt = yt + F * LDT;
-    bf16x8 zf[4];
+    u32x4 zf[4];
 #pragma unroll
     for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * w + c, 2 * u + hh));
 #pragma unroll
@@ -474,8 +504,7 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
       for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
 #pragma unroll
       for (int u = 0; u < 4; ++u)
-        st[T] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u],
-                                                        st[T], 0, 0, 0);
+        st[T] = E::mfma(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
     }
     if (more) fill_lds((it + 1) & 1);
     __syncthreads();
@@ -506,70 +535,81 @@ int raise_lds(K kernel) {
   return (int)e;
 }
 
-template <bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS>
 int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
                  void *out, const Geom &g, hipStream_t st) {
-  int rc = raise_lds(la_apply<REV, TRANS>);
+  int rc = raise_lds(la_apply<E, REV, TRANS>);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply<REV, TRANS><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
-                                                      (const bf16_t *)z, s, states, (bf16_t *)out, g);
+  la_apply<E, REV, TRANS><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
+                                                         (const bf16_t *)z, s, states, (bf16_t *)out, g);
   return (int)hipGetLastError();
 }
 
+template <class E>
 int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                 hipStream_t st) {
-  int rc = raise_lds(la_bwd3);
+  int rc = raise_lds(la_bwd3<E>);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3<<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k, (const bf16_t *)a.v,
-                                         (const bf16_t *)a.d_o, a.s, kv_states, dkv_states,
-                                         (bf16_t *)a.dq, (bf16_t *)a.dk, (bf16_t *)a.dv, g);
+  la_bwd3<E><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k, (const bf16_t *)a.v,
+                                            (const bf16_t *)a.d_o, a.s, kv_states, dkv_states,
+                                            (bf16_t *)a.dq, (bf16_t *)a.dk, (bf16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
 // segment it visits last (whose own state feeds nothing else) is skipped.
-template <bool REV>
+template <class E, bool REV>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g, skip_seg);
+  la_seg_state<E, REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g, skip_seg);
   return (int)hipGetLastError();
 }
 
-}  // namespace
-
-int mfma_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
+template <class E>
+int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, false>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
-  return launch_apply<false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
+  return launch_apply<E, false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
 }
 
-int mfma_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
+template <class E>
+int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
+    if ((rc = launch_state<E, false>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<true>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, true>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  return launch_bwd3(a, kv_states, dkv_states, g, st);
+  return launch_bwd3<E>(a, kv_states, dkv_states, g, st);
+}
+
+}  // namespace
+
+int mfma_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
+  return dtype == LASP_DTYPE_F16 ? fwd_e<ElemF16>(a, g, st) : fwd_e<ElemBF16>(a, g, st);
+}
+
+int mfma_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
+  return dtype == LASP_DTYPE_F16 ? bwd_e<ElemF16>(a, g, st) : bwd_e<ElemBF16>(a, g, st);
 }
 
 }  // namespace lasp

@@ -52,8 +52,8 @@ def test_generic_fp32_small(gpu_device, shape, state):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_generic_low_precision_io(gpu_device, dtype):
-    # n < 64 (bf16) and fp16 keep these on the generic kernels
-    inp = make_inputs(2, 12, 500 if dtype == torch.float16 else 50, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    # n < 64 keeps 16-bit I/O on the generic kernels
+    inp = make_inputs(2, 12, 50, 128, 64, dtype, seed=3, state=True, state_std=1.0)
     s = O.slopes_alibi(12)
     got = run_abi(inp, s, gpu_device)
     check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
@@ -171,3 +171,20 @@ def test_ragged_bf16_length_is_split_head_mfma_tail_generic(gpu_device, n, d, e)
         got = run_abi(inp, s, gpu_device, cache=cache)
         assert got["o"].shape == inp["v"].shape and got["dq"].shape == inp["q"].shape
         check(got, ref, 2e-2, what=f"ragged n={n} d={d} e={e} cache={cache}")
+
+
+@pytest.mark.parametrize("b,h,n,seg,state", [(1, 2, 256, 64, True), (2, 3, 1024, 256, True), (1, 4, 512, 0, False)])
+def test_mfma_fp16(gpu_device, b, h, n, seg, state):
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(b, h, n, 128, 128, torch.float16) == _abi.PATH_MFMA
+    inp = make_inputs(b, h, n, 128, 128, torch.float16, seed=n + 7, state=state, state_std=1.0)
+    s = O.slopes_baseline(h)
+    got = run_abi(inp, s, gpu_device, seg_len=seg)
+    check(got, oracle(inp, s), 2e-2, what=f"fp16 mfma b={b} h={h} n={n}")
+
+
+def test_fp16_narrow_and_ragged(gpu_device):
+    inp = make_inputs(1, 3, 333, 64, 96, torch.float16, seed=17, state=True, state_std=1.0)
+    s = O.slopes_alibi(3)
+    check(run_abi(inp, s, gpu_device), oracle(inp, s), 2e-2, what="fp16 ragged narrow")
