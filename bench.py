@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
 One step = forward + backward of causal decayed linear attention through the
-public operator (lightning_attn + autograd) on BASELINE configuration 2:
+public operator (lightning_attn + autograd) on the headline workload (TNL-1B head shape):
 b=1, h=16, n=65536, d=e=128, bf16, Q/K/V/dO ~ N(0,1)/sqrt(d), slopes
 2^(-8(i+1)/16); inputs are resident in HBM before the timed region.
 Prints ONE JSON line (metric = fwd+bwd tokens/s) that also carries
@@ -174,7 +174,7 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": "BASELINE config 2: lightning_attn fwd+bwd, b=1 h=16 n=65536 d=e=128, single pass, no KV state",
+            "workload": "TNL-1B attention head shape: lightning_attn fwd+bwd, b=1 h=16 n=65536 d=e=128, single pass, no KV state",
             "seg_len": seg_len,
             "n_seg": n_seg,
         },

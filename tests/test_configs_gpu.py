@@ -1,4 +1,4 @@
-"""BASELINE configurations 2-4 at full size on the GPU.
+"""The large benchmark configurations (2: TNL-1B head shape, 3: TNL-7B chunk, 4: 1M tokens) at full size.
 
 Where the fp64/fp32 oracle on every head would take too long on the host, the
 oracle is run on a subset of heads (stated per test) and the rest is covered by

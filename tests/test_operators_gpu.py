@@ -1,5 +1,5 @@
 """The public operators (autograd Functions + loopback state passing) against the
-oracle, at the BASELINE configurations or scaled-down versions of them.
+oracle, at the benchmark configurations or scaled-down versions of them.
 
 Tolerance: max|x - ref| / max|ref| <= 2e-2 for bf16 I/O (1e-3 for fp32)."""
 import pytest
@@ -82,7 +82,7 @@ def test_chain_matches_single_pass_and_oracle_small(gpu_device, op_name):
 
 
 def test_config1_chunk_chain_bf16(gpu_device):
-    """BASELINE config 1: b=2 h=12 d=128, n=16384 as 8 chunks of 2048 with KV / DKV carry."""
+    """Configuration 1 (SP=8 emulated on one GPU): b=2 h=12 d=128, n=16384 as 8 chunks of 2048 with KV / DKV carry."""
     inp = make_inputs(2, 12, 16384, 128, 128, torch.bfloat16, seed=1, state=False)
     s = O.slopes_baseline(12)
     ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s, inp["do"], dtype=torch.float32)

@@ -85,7 +85,7 @@ def test_segment_length_does_not_change_result(gpu_device):
 
 
 def test_config0_fp32_full(gpu_device):
-    """BASELINE config 0: b=2 n=2048 h=12 d=128 fp32, no incoming state."""
+    """Configuration 0 (the CPU-runnable case): b=2 n=2048 h=12 d=128 fp32, no incoming state."""
     inp = make_inputs(2, 12, 2048, 128, 128, torch.float32, seed=0, state=False)
     s = O.slopes_baseline(12)
     got = run_abi(inp, s, gpu_device)
