@@ -220,7 +220,7 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
 # states, so the results are exact, and the call runs an order of magnitude faster than on
 # the generic fp32-FMA kernels.  Everything else goes to the library unchanged.
 _MFMA_F = 128
-_MFMA_DTYPES = (torch.bfloat16, torch.float16)
+_MFMA_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
 
 
 def _pad_to_mfma(q, v) -> bool:

@@ -95,6 +95,9 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
 bool mfma_eligible(const Geom &g, int dtype) {
   return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && g.d == 128 && g.e == 128 && g.n % 64 == 0;
 }
+bool mfma_f32_eligible(const Geom &g, int dtype) {
+  return dtype == LASP_DTYPE_F32 && g.d == 128 && g.e == 128 && g.n % 32 == 0;
+}
 
 size_t state_bytes_of(const Geom &g) {
   return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.d * g.e;
@@ -179,7 +182,7 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
   Geom g;
   int rc = make_geom(b, h, n, d, e, dtype, 0, &g);
   if (rc) return rc;
-  return mfma_eligible(g, dtype) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
+  return (mfma_eligible(g, dtype) || mfma_f32_eligible(g, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
 }
 
 int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, const float *kv_in,
@@ -199,7 +202,9 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
   }
   FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype) ? mfma_fwd(a, g, dtype, st) : generic_fwd(a, g, dtype, st);
+  rc = mfma_eligible(g, dtype)       ? mfma_fwd(a, g, dtype, st)
+       : mfma_f32_eligible(g, dtype) ? mfma_f32_fwd(a, g, st)
+                                     : generic_fwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_fwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }
@@ -236,7 +241,9 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
   }
   if (need_kv) a.ws_kv = wp;
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype) ? mfma_bwd(a, g, dtype, st) : generic_bwd(a, g, dtype, st);
+  rc = mfma_eligible(g, dtype)       ? mfma_bwd(a, g, dtype, st)
+       : mfma_f32_eligible(g, dtype) ? mfma_f32_bwd(a, g, st)
+                                     : generic_bwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_bwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }

@@ -82,6 +82,8 @@ int generic_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st);
 int generic_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st);
 int mfma_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st);  // bf16 or fp16
 int mfma_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st);
+int mfma_f32_fwd(const FwdArgs &a, const Geom &g, hipStream_t st);
+int mfma_f32_bwd(const BwdArgs &a, const Geom &g, hipStream_t st);
 
 // The decayed scan over segment states is shared by both kernel families.
 //   forward  (reverse = 0): states[seg] <- state entering segment seg from the

@@ -32,7 +32,8 @@ def test_library_loaded_and_path_selection(gpu_device):
     lib = _abi.load()
     assert lib.lasp_abi_version() == 1
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
-    assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_MFMA
+    assert _abi.kernel_path(2, 12, 2048, 128, 96, torch.float32) == _abi.PATH_GENERIC
     assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_GENERIC
     assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_GENERIC
 
@@ -40,7 +41,7 @@ def test_library_loaded_and_path_selection(gpu_device):
 @pytest.mark.parametrize("state", [False, True])
 @pytest.mark.parametrize("shape", [
     (1, 2, 64, 32, 32, 0), (2, 3, 200, 64, 32, 0), (1, 2, 7, 16, 48, 0),
-    (1, 2, 1024, 128, 128, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0),
+    (1, 2, 1024, 128, 96, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0), (1, 2, 40, 128, 128, 0),
 ])
 def test_generic_fp32_small(gpu_device, shape, state):
     b, h, n, d, e, seg = shape
@@ -188,3 +189,31 @@ def test_fp16_narrow_and_ragged(gpu_device):
     inp = make_inputs(1, 3, 333, 64, 96, torch.float16, seed=17, state=True, state_std=1.0)
     s = O.slopes_alibi(3)
     check(run_abi(inp, s, gpu_device), oracle(inp, s), 2e-2, what="fp16 ragged narrow")
+
+
+# ---------------------------------------------------------------- fp32 MFMA kernels (d = e = 128)
+@pytest.mark.parametrize("state", [False, True])
+@pytest.mark.parametrize("b,h,n,seg", [
+    (1, 1, 32, 0), (1, 2, 96, 64), (1, 2, 256, 64), (2, 3, 512, 128), (1, 4, 1024, 256), (1, 2, 2048, 2048),
+    (2, 2, 320, 256), (3, 5, 192, 128),
+])
+def test_mfma_fp32(gpu_device, b, h, n, seg, state):
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(b, h, n, 128, 128, torch.float32) == _abi.PATH_MFMA
+    inp = make_inputs(b, h, n, 128, 128, torch.float32, seed=n + h + 1, state=state, state_std=1.0)
+    s = O.slopes_baseline(h) if h > 1 else torch.tensor([0.05])
+    got = run_abi(inp, s, gpu_device, seg_len=seg)
+    check(got, oracle(inp, s), 1e-4, what=f"fp32 mfma b={b} h={h} n={n} seg={seg} state={state}")
+
+
+def test_mfma_fp32_special_slopes_and_padding(gpu_device):
+    inp = make_inputs(1, 3, 512, 128, 128, torch.float32, seed=31, state=True, state_std=1.0)
+    s = torch.tensor([0.0, 1.0, 30.0])
+    got = run_abi(inp, s, gpu_device, seg_len=128)
+    assert all(torch.isfinite(v_).all() for v_ in got.values())
+    check(got, oracle(inp, s), 1e-4, what="fp32 mfma s in {0, 1, 30}")
+    # narrow heads and a ragged length reach the same kernels through padding / splitting
+    inp = make_inputs(1, 2, 300, 64, 96, torch.float32, seed=32, state=True, state_std=1.0)
+    s = O.slopes_baseline(2)
+    check(run_abi(inp, s, gpu_device), oracle(inp, s), 1e-4, what="fp32 narrow ragged")
