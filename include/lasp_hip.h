@@ -55,7 +55,7 @@ extern "C" {
 
 /* Which kernel family a shape/dtype is served by (lasp_kernel_path). */
 #define LASP_PATH_GENERIC 0 /* fp32-FMA kernels: any dtype, any n, d,e <= 128 */
-#define LASP_PATH_MFMA 1    /* MFMA kernels, d = e = 128: bf16 / fp16 with n % 64 == 0, fp32 with n % 32 == 0 */
+#define LASP_PATH_MFMA 1    /* MFMA kernels: d = e = 128, any dtype, any n (a ragged tail is masked) */
 
 int lasp_abi_version(void);
 

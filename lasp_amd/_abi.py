@@ -214,18 +214,17 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
 
 
 # ---------------------------------------------------------------------------------------
-# Narrow heads on the MFMA kernels.  The bf16 MFMA kernels take d = e = 128 only.  A bf16
-# call with narrower features (the reference's own test uses e = 64, tests/test.py:95) is
-# zero-padded to 128 here: zero feature columns add nothing to q.k, to the outputs or to the
-# states, so the results are exact, and the call runs an order of magnitude faster than on
-# the generic fp32-FMA kernels.  Everything else goes to the library unchanged.
+# Narrow heads on the MFMA kernels.  The MFMA kernels take d = e = 128 only.  A call with
+# narrower features (the reference's own test uses e = 64, tests/test.py:95) is zero-padded
+# to 128 here: zero feature columns add nothing to q.k, to the outputs or to the states, so the
+# results are exact, and the call runs an order of magnitude faster than on the generic
+# fp32-FMA kernels.  Everything else goes to the library unchanged.
 _MFMA_F = 128
-_MFMA_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
 
 
 def _pad_to_mfma(q, v) -> bool:
-    n, d, e = q.shape[2], q.shape[3], v.shape[3]
-    return q.dtype in _MFMA_DTYPES and n % 64 == 0 and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
+    d, e = q.shape[3], v.shape[3]
+    return q.dtype in DTYPE_CODE and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
 
 
 def _pad_last(t, size):
@@ -240,33 +239,9 @@ def _pad_state(t, d, e):
     return out
 
 
-def _ragged_for_mfma(q, v) -> bool:
-    n, d, e = q.shape[2], q.shape[3], v.shape[3]
-    return q.dtype in _MFMA_DTYPES and n % 64 != 0 and n > 64 and d <= _MFMA_F and e <= _MFMA_F
-
-
-# A bf16 chunk whose length is not a multiple of 64 is cut at the last multiple: the head runs
-# on the MFMA kernels, the tail (< 64 tokens) on the generic ones, and the d x e state is
-# carried across the cut exactly as between two chunks of a sequence-parallel chain.  The
-# state at the cut is what such a call hands back as `seg_states` (4-D instead of 5-D).
-def _split_ragged(t, n64):
-    return t[:, :, :n64].contiguous(), t[:, :, n64:].contiguous()
-
-
 def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
-    """Forward of one chunk: (o, seg_states, seg_len).  See _chunk_fwd_exact.  Narrow bf16 heads
-    are zero-padded and ragged bf16 lengths are split so that the MFMA kernels do the bulk."""
-    if q.dim() != 4 or v.dim() != 4:
-        return _chunk_fwd_exact(q, k, v, s, kv_in, kv_out, seg_len)
-    if _ragged_for_mfma(q, v):
-        b, h, n, d, e = _shapes(q, k, v)
-        n64 = n // 64 * 64
-        (q1, q2), (k1, k2), (v1, v2) = (_split_ragged(t, n64) for t in (q, k, v))
-        kv_mid = torch.empty(b, h, d, e, dtype=torch.float32, device=q.device)
-        o1, _, seg_len = chunk_fwd(q1, k1, v1, s, kv_in, kv_mid, seg_len)
-        o2, _, _ = _chunk_fwd_exact(q2, k2, v2, s, kv_mid, kv_out, 0)
-        return torch.cat([o1, o2], dim=2), kv_mid, seg_len
-    if not _pad_to_mfma(q, v):
+    """Forward of one chunk: (o, seg_states, seg_len).  See _chunk_fwd_exact; narrow heads are padded."""
+    if q.dim() != 4 or v.dim() != 4 or not _pad_to_mfma(q, v):
         return _chunk_fwd_exact(q, k, v, s, kv_in, kv_out, seg_len)
     b, h, n, d, e = _shapes(q, k, v)
     _check_state("kv_in", kv_in, b, h, d, e)
@@ -280,23 +255,9 @@ def chunk_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
 
 
 def chunk_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):
-    """Backward of one chunk: (dq, dk, dv).  See _chunk_bwd_exact; kv_seg_states, if given, must be
-    what chunk_fwd returned for the same inputs."""
-    if q.dim() != 4 or v.dim() != 4:
-        return _chunk_bwd_exact(q, k, v, s, do, kv_in, dkv_in, dkv_out, kv_seg_states, seg_len)
-    if _ragged_for_mfma(q, v):
-        b, h, n, d, e = _shapes(q, k, v)
-        n64 = n // 64 * 64
-        (q1, q2), (k1, k2), (v1, v2), (do1, do2) = (_split_ragged(t, n64) for t in (q, k, v, do))
-        kv_mid = kv_seg_states
-        if kv_mid is None:  # the state at the cut was not kept: run the head's forward again
-            kv_mid = torch.empty(b, h, d, e, dtype=torch.float32, device=q.device)
-            chunk_fwd(q1, k1, v1, s, kv_in, kv_mid, seg_len)
-        dkv_mid = torch.empty(b, h, d, e, dtype=torch.float32, device=q.device)
-        dq2, dk2, dv2 = _chunk_bwd_exact(q2, k2, v2, s, do2, kv_mid, dkv_in, dkv_mid, None, 0)
-        dq1, dk1, dv1 = chunk_bwd(q1, k1, v1, s, do1, kv_in, dkv_mid, dkv_out, None, seg_len)
-        return torch.cat([dq1, dq2], 2), torch.cat([dk1, dk2], 2), torch.cat([dv1, dv2], 2)
-    if not _pad_to_mfma(q, v):
+    """Backward of one chunk: (dq, dk, dv).  See _chunk_bwd_exact; narrow heads are padded
+    (kv_seg_states must then be what chunk_fwd returned for the same call)."""
+    if q.dim() != 4 or v.dim() != 4 or not _pad_to_mfma(q, v):
         return _chunk_bwd_exact(q, k, v, s, do, kv_in, dkv_in, dkv_out, kv_seg_states, seg_len)
     b, h, n, d, e = _shapes(q, k, v)
     _check_state("kv_in", kv_in, b, h, d, e)

@@ -93,10 +93,10 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
 }
 
 bool mfma_eligible(const Geom &g, int dtype) {
-  return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && g.d == 128 && g.e == 128 && g.n % 64 == 0;
+  return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && g.d == 128 && g.e == 128;
 }
 bool mfma_f32_eligible(const Geom &g, int dtype) {
-  return dtype == LASP_DTYPE_F32 && g.d == 128 && g.e == 128 && g.n % 32 == 0;
+  return dtype == LASP_DTYPE_F32 && g.d == 128 && g.e == 128;
 }
 
 size_t state_bytes_of(const Geom &g) {

@@ -1,4 +1,5 @@
-// bf16 / fp16 MFMA kernels for d = e = 128, n % 64 == 0 (gfx950, wave64).
+// bf16 / fp16 MFMA kernels for d = e = 128 (gfx950, wave64); a chunk length that is not a
+// multiple of 64 ends in one partial block (RAGGED instantiations).
 //
 // One kernel, `la_apply`, evaluates a causal (or anti-causal) decayed linear
 // attention over a segment of 64-token blocks given the state entering it:
@@ -185,7 +186,8 @@ __device__ __forceinline__ u32x4 load_row_pieces(const u32x2 *row, const LoaderR
 struct SegWork {
   int bh, seg;
   int64_t tok0;  // first token of the segment
-  int nblk;      // 64-token blocks in it
+  int nblk;      // 64-token blocks in it, the last one possibly partial
+  int tail;      // tokens in its last block (1..64); below 64 only at the end of a ragged chunk
 };
 // `item` enumerates (b*h, segment) pairs
 __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
@@ -195,12 +197,16 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
   r.tok0 = (int64_t)r.seg * g.seg_len;
   int64_t t1 = r.tok0 + g.seg_len;
   if (t1 > g.n) t1 = g.n;
-  r.nblk = (int)((t1 - r.tok0) / BLK);
+  const int tokens = (int)(t1 - r.tok0);
+  r.nblk = (tokens + BLK - 1) / BLK;
+  r.tail = tokens - (r.nblk - 1) * BLK;
   return r;
 }
 
 // ------------------------------------------------------------------------------
-template <class E, bool REV, bool TRANS>
+// RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
+// partial; the aligned instantiation carries none of that bookkeeping.
+template <class E, bool REV, bool TRANS, bool RAGGED>
 __device__ __forceinline__ void
 apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
@@ -257,14 +263,31 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 
   // ---- block loader: registers <- global, LDS <- registers
   u32x4 nx[4], ny[4], nz[4];
+  // a partial block (the end of a ragged chunk) reads its missing rows as zeros
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
     const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units (32 per row)
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    if (!RAGGED || len == BLK) {
 #pragma unroll
-    for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
+      for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
-      nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
+      for (int r = 0; r < 4; ++r) {
+        ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
+        nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
+      }
+    } else {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int row = xr.rowq + 16 * it;
+        nx[it] = row < len ? load_row_pieces(Xg + off + row * 32, xr) : zero;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 4 * yr.rowq + r;
+        ny[r] = row < len ? load_row_pieces(Yg + off + row * 32, yr) : zero;
+        nz[r] = row < len ? load_row_pieces(Zg + off + row * 32, yr) : zero;
+      }
     }
   };
   auto fill_lds = [&]() __attribute__((always_inline)) {
@@ -287,6 +310,16 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
   for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
+    // A partial block is the chunk's last one.  Going forwards nothing after it uses the state;
+    // going backwards it comes first and the entering state sits `len` (not 64) tokens ahead.
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    float qd[2] = {qdec[0], qdec[1]};
+    float bd = blockdec;
+    if (RAGGED && REV && len != BLK) {
+      qd[0] = decay(sl, (float)max(len - c, 0));
+      qd[1] = decay(sl, (float)max(len - 32 - c, 0));
+      bd = decay(sl, (float)len);
+    }
 
     // (1) one sweep over the 8 feature steps feeds two products from the same X fragments:
     //     state term, transposed:  acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
@@ -342,12 +375,12 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 #pragma unroll
     for (int I = 0; I < 2; ++I)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[I][r] *= qdec[I];
+      for (int r = 0; r < 16; ++r) acc[I][r] *= qd[I];
     // the state has been consumed by the sweep: decay it now, ahead of the update in (4)
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 
     __syncthreads();  // A: score tile complete; XN / YN no longer read
 
@@ -392,8 +425,9 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int row = rowq + 16 * r4;
-        __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(smem + OFF_YN + row * LDN + chunk * 16),
-                                    &Og[off + row * 16 + chunk]);
+        if (!RAGGED || row < len)
+          __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(smem + OFF_YN + row * LDN + chunk * 16),
+                                      &Og[off + row * 16 + chunk]);
       }
     }
     if (more) {
@@ -404,20 +438,20 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
   }
 }
 
-template <class E, bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
          const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
          Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<E, REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
+  apply_body<E, REV, TRANS, RAGGED>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
 // work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
 // the triple is spread over block indices 8 apart so that all three land on the same
 // XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
-template <class E>
+template <class E, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
         const bf16_t *__restrict__ DO, const float *__restrict__ S,
@@ -430,17 +464,17 @@ la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    apply_body<E, false, true>(DO, V, K, S, kv_states, DQ, g, item, smem);
+    apply_body<E, false, true, RAGGED>(DO, V, K, S, kv_states, DQ, g, item, smem);
   else if (role == 1)
-    apply_body<E, true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem);
+    apply_body<E, true, false, RAGGED>(K, Q, DO, S, dkv_states, DV, g, item, smem);
   else
-    apply_body<E, true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem);
+    apply_body<E, true, true, RAGGED>(V, DO, Q, S, dkv_states, DK, g, item, smem);
 }
 
 // ------------------------------------------------------------------------------
 // A segment's own state:  causal  sum_b l^(L-b) y_b^T z_b ;  anti-causal  sum_b l^b y_b^T z_b
 // (b from the segment start, L its length), written token-free as 128 x 128 fp32.
-template <class E, bool REV>
+template <class E, bool REV, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
@@ -471,28 +505,44 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
 
+  // A partial block (the end of a ragged chunk) reads its missing rows as zeros; going
+  // forwards it is the last block, and its tokens sit `len - b` (not 64 - b) before the
+  // segment end.
   u32x4 ny[4], nz[4];
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
     const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
-      nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
+      const int row = 4 * yr.rowq + r;
+      ny[r] = (!RAGGED || row < len) ? load_row_pieces(Yg + off + row * 32, yr) : zero;
+      nz[r] = (!RAGGED || row < len) ? load_row_pieces(Zg + off + row * 32, yr) : zero;
     }
   };
-  auto fill_lds = [&](int buf) __attribute__((always_inline)) {
-    store_transposed<E, true>(smem[buf], ny, yr, kdec);
+  auto fill_lds = [&](int buf, int blk) __attribute__((always_inline)) {
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    if (RAGGED && !REV && len != BLK) {
+      float kd[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
+      store_transposed<E, true>(smem[buf], ny, yr, kd);
+    } else {
+      store_transposed<E, true>(smem[buf], ny, yr, kdec);
+    }
     store_transposed<E, false>(smem[buf] + F * LDT, nz, yr, kdec);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
   const int step = REV ? -1 : 1;
   issue_loads(first);
-  fill_lds(0);
+  fill_lds(0, first);
   __syncthreads();
   for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
     const char *yt = smem[it & 1];
     const char *zt = yt + F * LDT;
     u32x4 zf[4];
@@ -501,12 +551,12 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
 #pragma unroll
     for (int T = 0; T < 4; ++T) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         st[T] = E::mfma(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
     }
-    if (more) fill_lds((it + 1) & 1);
+    if (more) fill_lds((it + 1) & 1, blk + step);
     __syncthreads();
   }
 
@@ -535,81 +585,88 @@ int raise_lds(K kernel) {
   return (int)e;
 }
 
-template <class E, bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS, bool RAGGED>
 int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
                  void *out, const Geom &g, hipStream_t st) {
-  int rc = raise_lds(la_apply<E, REV, TRANS>);
+  int rc = raise_lds(la_apply<E, REV, TRANS, RAGGED>);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply<E, REV, TRANS><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
-                                                         (const bf16_t *)z, s, states, (bf16_t *)out, g);
+  la_apply<E, REV, TRANS, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
+                                                                 (const bf16_t *)z, s, states,
+                                                                 (bf16_t *)out, g);
   return (int)hipGetLastError();
 }
 
-template <class E>
+template <class E, bool RAGGED>
 int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                 hipStream_t st) {
-  int rc = raise_lds(la_bwd3<E>);
+  int rc = raise_lds(la_bwd3<E, RAGGED>);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3<E><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k, (const bf16_t *)a.v,
-                                            (const bf16_t *)a.d_o, a.s, kv_states, dkv_states,
-                                            (bf16_t *)a.dq, (bf16_t *)a.dk, (bf16_t *)a.dv, g);
+  la_bwd3<E, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k,
+                                                    (const bf16_t *)a.v, (const bf16_t *)a.d_o, a.s,
+                                                    kv_states, dkv_states, (bf16_t *)a.dq,
+                                                    (bf16_t *)a.dk, (bf16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
 // segment it visits last (whose own state feeds nothing else) is skipped.
-template <class E, bool REV>
+template <class E, bool REV, bool RAGGED>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g, skip_seg);
+  la_seg_state<E, REV, RAGGED><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g,
+                                                      skip_seg);
   return (int)hipGetLastError();
 }
 
-template <class E>
+template <class E, bool RAGGED>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
-    if ((rc = launch_state<E, false>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, false, RAGGED>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
-  return launch_apply<E, false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
+  return launch_apply<E, false, false, RAGGED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
 }
 
-template <class E>
+template <class E, bool RAGGED>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<E, false>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
+    if ((rc = launch_state<E, false, RAGGED>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<E, true>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, true, RAGGED>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  return launch_bwd3<E>(a, kv_states, dkv_states, g, st);
+  return launch_bwd3<E, RAGGED>(a, kv_states, dkv_states, g, st);
 }
 
 }  // namespace
 
 int mfma_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
-  return dtype == LASP_DTYPE_F16 ? fwd_e<ElemF16>(a, g, st) : fwd_e<ElemBF16>(a, g, st);
+  const bool ragged = g.n % BLK != 0;
+  if (dtype == LASP_DTYPE_F16) return ragged ? fwd_e<ElemF16, true>(a, g, st) : fwd_e<ElemF16, false>(a, g, st);
+  return ragged ? fwd_e<ElemBF16, true>(a, g, st) : fwd_e<ElemBF16, false>(a, g, st);
 }
 
 int mfma_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
-  return dtype == LASP_DTYPE_F16 ? bwd_e<ElemF16>(a, g, st) : bwd_e<ElemBF16>(a, g, st);
+  const bool ragged = g.n % BLK != 0;
+  if (dtype == LASP_DTYPE_F16) return ragged ? bwd_e<ElemF16, true>(a, g, st) : bwd_e<ElemF16, false>(a, g, st);
+  return ragged ? bwd_e<ElemBF16, true>(a, g, st) : bwd_e<ElemBF16, false>(a, g, st);
 }
 
 }  // namespace lasp

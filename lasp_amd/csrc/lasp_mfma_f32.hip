@@ -1,4 +1,4 @@
-// fp32 MFMA kernels for d = e = 128, n % 32 == 0 (gfx950, wave64): the same decomposition
+// fp32 MFMA kernels for d = e = 128 (gfx950, wave64): the same decomposition
 // as the 16-bit kernels -- one routine evaluates a causal or anti-causal decayed linear
 // attention over a segment given the state entering it, and the four outputs of the
 // operator are instances of it (O: x=Q y=K z=V; dQ: x=dO y=V z=K with the state transposed;
@@ -54,7 +54,8 @@ __device__ __forceinline__ int tr_off(int f, int g16) {
 struct SegWork {
   int bh, seg;
   int64_t tok0;
-  int nblk;  // 32-token blocks
+  int nblk;  // 32-token blocks, the last one possibly partial
+  int tail;  // tokens in the last block (1..32); below 32 only at the end of a ragged chunk
 };
 __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
   SegWork r;
@@ -63,7 +64,9 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
   r.tok0 = (int64_t)r.seg * g.seg_len;
   int64_t t1 = r.tok0 + g.seg_len;
   if (t1 > g.n) t1 = g.n;
-  r.nblk = (int)((t1 - r.tok0) / BLK);
+  const int tokens = (int)(t1 - r.tok0);
+  r.nblk = (tokens + BLK - 1) / BLK;
+  r.tail = tokens - (r.nblk - 1) * BLK;
   return r;
 }
 
@@ -82,7 +85,10 @@ __device__ __forceinline__ void store_transposed(char *tile, const f32x4 (&rows)
   }
 }
 
-template <bool REV, bool TRANS>
+// RAGGED: the chunk length is not a multiple of 32, so the last block of the last segment is
+// partial (missing rows read as zeros, stores masked, and -- going backwards, where that block
+// comes first -- the entering state sits `len` tokens ahead instead of 32).
+template <bool REV, bool TRANS, bool RAGGED>
 __device__ __forceinline__ void
 apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, float *__restrict__ Out,
@@ -133,12 +139,18 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
   f32x4 nx[4], ny[4], nz[4];
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
     const int64_t off = (int64_t)blk * (BLK * F / 4);  // 16-byte units, 32 per row
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int it = 0; it < 4; ++it) nx[it] = Xg[off + (rq + 8 * it) * 32 + cq];
+    for (int it = 0; it < 4; ++it) {
+      const int row = rq + 8 * it;
+      nx[it] = (!RAGGED || row < len) ? Xg[off + row * 32 + cq] : zero;
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      ny[r] = Yg[off + (4 * rq + r) * 32 + cq];
-      nz[r] = Zg[off + (4 * rq + r) * 32 + cq];
+      const int row = 4 * rq + r;
+      ny[r] = (!RAGGED || row < len) ? Yg[off + row * 32 + cq] : zero;
+      nz[r] = (!RAGGED || row < len) ? Zg[off + row * 32 + cq] : zero;
     }
   };
   auto fill_lds = [&]() __attribute__((always_inline)) {
@@ -161,6 +173,12 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
   for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    float qd = qdec, bd = blockdec;
+    if (RAGGED && REV && len != BLK) {
+      qd = decay(sl, (float)max(len - c, 0));
+      bd = decay(sl, (float)len);
+    }
 
     // (1) sweep over the features: state term and score tile from the same X elements
     //     acc[4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f]      (a = c)
@@ -191,7 +209,7 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
       const int b = 8 * (r >> 2) + 4 * hh + (r & 3);
       const int dist = REV ? b - c : c - b;
       sc[r] = dist >= 0 ? sc[r] * decay(sl, (float)dist) : 0.f;
-      acc[r] *= qdec;
+      acc[r] *= qd;
     }
     // (3) intra-block term and (4) state update share the Z^T elements
     f32x4 zf[4];
@@ -204,7 +222,7 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
 #pragma unroll
     for (int T = 0; T < 4; ++T) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         const f32x4 yt = lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * gq + hh));
@@ -213,7 +231,7 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
       }
     }
     // (5) output: lane (c, hh) holds, for token c, four consecutive columns per g
-    {
+    if (!RAGGED || c < len) {
       float *orow = Og + ((int64_t)blk * BLK + c) * F + 32 * w + 4 * hh;
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
@@ -233,16 +251,17 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
   }
 }
 
-template <bool REV, bool TRANS>
+template <bool REV, bool TRANS, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la32_apply(const float *__restrict__ X, const float *__restrict__ Y, const float *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, float *__restrict__ Out, Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
+  apply_body<REV, TRANS, RAGGED>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
 }
 
 // dQ, dV and dK in one launch; the three workgroups of a (b*h, segment) sit 8 block indices
 // apart, i.e. on the same XCD
+template <bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la32_bwd3(const float *__restrict__ Q, const float *__restrict__ K, const float *__restrict__ V,
           const float *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_states,
@@ -255,15 +274,15 @@ la32_bwd3(const float *__restrict__ Q, const float *__restrict__ K, const float 
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    apply_body<false, true>(DO, V, K, S, kv_states, DQ, g, item, smem);
+    apply_body<false, true, RAGGED>(DO, V, K, S, kv_states, DQ, g, item, smem);
   else if (role == 1)
-    apply_body<true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem);
+    apply_body<true, false, RAGGED>(K, Q, DO, S, dkv_states, DV, g, item, smem);
   else
-    apply_body<true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem);
+    apply_body<true, true, RAGGED>(V, DO, Q, S, dkv_states, DK, g, item, smem);
 }
 
 // a segment's own state: causal sum_b l^(L-b) y_b^T z_b ; anti-causal sum_b l^b y_b^T z_b
-template <bool REV>
+template <bool REV, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
 la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const float *__restrict__ S,
                float *__restrict__ states, Geom g, int skip_seg) {
@@ -297,25 +316,39 @@ la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const f
   f32x4 ny[4], nz[4];
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
     const int64_t off = (int64_t)blk * (BLK * F / 4);
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      ny[r] = Yg[off + (4 * rq + r) * 32 + cq];
-      nz[r] = Zg[off + (4 * rq + r) * 32 + cq];
+      const int row = 4 * rq + r;
+      ny[r] = (!RAGGED || row < len) ? Yg[off + row * 32 + cq] : zero;
+      nz[r] = (!RAGGED || row < len) ? Zg[off + row * 32 + cq] : zero;
     }
   };
-  auto fill_lds = [&](int buf) __attribute__((always_inline)) {
-    store_transposed(smem[buf], ny, cq, rq, kdec);
+  // going forwards a partial block is the last one: its tokens sit `len - b` before the segment end
+  auto fill_lds = [&](int buf, int blk) __attribute__((always_inline)) {
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    if (RAGGED && !REV && len != BLK) {
+      float kd[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * rq + r), 0));
+      store_transposed(smem[buf], ny, cq, rq, kd);
+    } else {
+      store_transposed(smem[buf], ny, cq, rq, kdec);
+    }
     store_transposed(smem[buf] + F * LDT, nz, cq, rq, ones);
   };
 
   const int first = REV ? sw.nblk - 1 : 0;
   const int step = REV ? -1 : 1;
   issue_loads(first);
-  fill_lds(0);
+  fill_lds(0, first);
   __syncthreads();
   for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
+    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
     const char *ytile = smem[it & 1];
     const char *ztile = ytile + F * LDT;
     f32x4 zf[4];
@@ -324,7 +357,7 @@ la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const f
 #pragma unroll
     for (int T = 0; T < 4; ++T) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         const f32x4 yt = lds16(ytile + tr_off(32 * T + c, 2 * gq + hh));
@@ -332,7 +365,7 @@ la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const f
         for (int r = 0; r < 4; ++r) st[T] = mfma(yt[r], zf[gq][r], st[T]);
       }
     }
-    if (more) fill_lds((it + 1) & 1);
+    if (more) fill_lds((it + 1) & 1, blk + step);
     __syncthreads();
   }
   float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
@@ -359,57 +392,68 @@ int raise_lds(K kernel) {
   return (int)e;
 }
 
-template <bool REV>
+template <bool REV, bool RAGGED>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la32_seg_state<REV><<<grid, NTHR, 0, st>>>((const float *)y, (const float *)z, s, states, g, skip_seg);
+  la32_seg_state<REV, RAGGED><<<grid, NTHR, 0, st>>>((const float *)y, (const float *)z, s, states, g,
+                                                     skip_seg);
+  return (int)hipGetLastError();
+}
+
+template <bool RAGGED>
+int fwd_r(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc;
+  const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
+  if (need_states) {
+    if ((rc = launch_state<false, RAGGED>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
+  }
+  if ((rc = raise_lds(la32_apply<false, false, RAGGED>))) return rc;
+  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_APPLY, st);
+  la32_apply<false, false, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const float *)a.q, (const float *)a.k,
+                                                                  (const float *)a.v, a.s,
+                                                                  need_states ? a.seg_states : nullptr,
+                                                                  (float *)a.o, g);
+  return (int)hipGetLastError();
+}
+
+template <bool RAGGED>
+int bwd_r(const BwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc;
+  const float *kv_states = a.kv_seg_states;
+  if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
+    if ((rc = launch_state<false, RAGGED>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
+    if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
+    kv_states = a.ws_kv;
+  }
+  const float *dkv_states = nullptr;
+  if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
+    if ((rc = launch_state<true, RAGGED>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
+    dkv_states = a.ws_dkv;
+  }
+  if ((rc = raise_lds(la32_bwd3<RAGGED>))) return rc;
+  const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
+  const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
+  ProfScope prof(KC_BWD3, st);
+  la32_bwd3<RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const float *)a.q, (const float *)a.k,
+                                                   (const float *)a.v, (const float *)a.d_o, a.s, kv_states,
+                                                   dkv_states, (float *)a.dq, (float *)a.dk, (float *)a.dv, g);
   return (int)hipGetLastError();
 }
 
 }  // namespace
 
 int mfma_f32_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc;
-  const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
-  if (need_states) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
-    if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
-  }
-  if ((rc = raise_lds(la32_apply<false, false>))) return rc;
-  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
-  ProfScope prof(KC_APPLY, st);
-  la32_apply<false, false><<<grid, NTHR, APPLY_LDS, st>>>((const float *)a.q, (const float *)a.k,
-                                                          (const float *)a.v, a.s,
-                                                          need_states ? a.seg_states : nullptr,
-                                                          (float *)a.o, g);
-  return (int)hipGetLastError();
+  return g.n % BLK != 0 ? fwd_r<true>(a, g, st) : fwd_r<false>(a, g, st);
 }
 
 int mfma_f32_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc;
-  const float *kv_states = a.kv_seg_states;
-  if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<false>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
-    if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
-    kv_states = a.ws_kv;
-  }
-  const float *dkv_states = nullptr;
-  if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<true>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
-    if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
-    dkv_states = a.ws_dkv;
-  }
-  if ((rc = raise_lds(la32_bwd3))) return rc;
-  const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
-  const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
-  ProfScope prof(KC_BWD3, st);
-  la32_bwd3<<<grid, NTHR, APPLY_LDS, st>>>((const float *)a.q, (const float *)a.k, (const float *)a.v,
-                                           (const float *)a.d_o, a.s, kv_states, dkv_states,
-                                           (float *)a.dq, (float *)a.dk, (float *)a.dv, g);
-  return (int)hipGetLastError();
+  return g.n % BLK != 0 ? bwd_r<true>(a, g, st) : bwd_r<false>(a, g, st);
 }
 
 }  // namespace lasp

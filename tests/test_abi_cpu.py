@@ -77,9 +77,9 @@ def test_kernel_path_selection(lib):
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.float16) == _abi.PATH_MFMA
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.float32) == _abi.PATH_MFMA
-    assert _abi.kernel_path(1, 16, 65520, 128, 128, torch.float32) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65520, 128, 128, torch.float32) == _abi.PATH_MFMA   # ragged: masked tail
     assert _abi.kernel_path(1, 16, 65536, 128, 64, torch.float32) == _abi.PATH_GENERIC
-    assert _abi.kernel_path(1, 16, 65500, 128, 128, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65500, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_GENERIC
 
 

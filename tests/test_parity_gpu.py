@@ -12,16 +12,22 @@ from tests.helpers import TOL, check, make_inputs, oracle
 pytestmark = pytest.mark.gpu
 
 
-def run_abi(inp, s, dev, seg_len=0, cache=False):
-    """One chunk forward + backward through lasp_amd._abi (ctypes -> liblasp_hip.so)."""
+def run_abi(inp, s, dev, seg_len=0, cache=False, exact=False):
+    """One chunk forward + backward through lasp_amd._abi (ctypes -> liblasp_hip.so).
+
+    exact=True hands the shape to the library as is (narrow heads then run on the generic
+    kernels); otherwise the Python layer zero-pads narrow heads onto the MFMA kernels."""
     from lasp_amd import _abi
+
+    fwd = _abi._chunk_fwd_exact if exact else _abi.chunk_fwd
+    bwd = _abi._chunk_bwd_exact if exact else _abi.chunk_bwd
 
     t = {k_: (x.to(dev) if x is not None else None) for k_, x in inp.items()}
     kv_out = torch.empty_like(t["kv"]) if t["kv"] is not None else None
     dkv_out = torch.empty_like(t["dkv"]) if t["dkv"] is not None else None
-    o, states, sl = _abi.chunk_fwd(t["q"], t["k"], t["v"], s, kv_in=t["kv"], kv_out=kv_out, seg_len=seg_len)
-    dq, dk, dv = _abi.chunk_bwd(t["q"], t["k"], t["v"], s, t["do"], kv_in=t["kv"], dkv_in=t["dkv"],
-                                dkv_out=dkv_out, kv_seg_states=states if cache else None, seg_len=sl)
+    o, states, sl = fwd(t["q"], t["k"], t["v"], s, kv_in=t["kv"], kv_out=kv_out, seg_len=seg_len)
+    dq, dk, dv = bwd(t["q"], t["k"], t["v"], s, t["do"], kv_in=t["kv"], dkv_in=t["dkv"],
+                     dkv_out=dkv_out, kv_seg_states=states if cache else None, seg_len=sl)
     torch.cuda.synchronize()
     return dict(o=o, kv_out=kv_out, dq=dq, dk=dk, dv=dv, dkv_out=dkv_out)
 
@@ -34,45 +40,45 @@ def test_library_loaded_and_path_selection(gpu_device):
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 96, torch.float32) == _abi.PATH_GENERIC
-    assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_GENERIC
 
 
 @pytest.mark.parametrize("state", [False, True])
 @pytest.mark.parametrize("shape", [
     (1, 2, 64, 32, 32, 0), (2, 3, 200, 64, 32, 0), (1, 2, 7, 16, 48, 0),
-    (1, 2, 1024, 128, 96, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0), (1, 2, 40, 128, 128, 0),
+    (1, 2, 1024, 128, 96, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0), (1, 2, 40, 96, 128, 0),
 ])
 def test_generic_fp32_small(gpu_device, shape, state):
     b, h, n, d, e, seg = shape
     inp = make_inputs(b, h, n, d, e, torch.float32, seed=n + d, state=state, state_std=1.0)
     s = O.slopes_baseline(h)
-    got = run_abi(inp, s, gpu_device, seg_len=seg)
+    got = run_abi(inp, s, gpu_device, seg_len=seg, exact=True)
     check(got, oracle(inp, s), 1e-3 if n > 64 else 2e-4, what=f"fp32 {shape} state={state}")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_generic_low_precision_io(gpu_device, dtype):
-    # n < 64 keeps 16-bit I/O on the generic kernels
-    inp = make_inputs(2, 12, 50, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    # e != d handed to the library as is: generic kernels with 16-bit I/O
+    inp = make_inputs(2, 12, 500, 128, 64, dtype, seed=3, state=True, state_std=1.0)
     s = O.slopes_alibi(12)
-    got = run_abi(inp, s, gpu_device)
+    got = run_abi(inp, s, gpu_device, exact=True)
     check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
 
 
 def test_special_slopes_zero_and_huge(gpu_device):
     inp = make_inputs(1, 2, 300, 32, 32, torch.float32, seed=5, state=True, state_std=1.0)
     s = torch.tensor([0.0, 50.0])
-    got = run_abi(inp, s, gpu_device)
+    got = run_abi(inp, s, gpu_device, exact=True)
     assert all(torch.isfinite(v_).all() for v_ in got.values())
     check(got, oracle(inp, s), 1e-3, what="s in {0, 50}")
 
 
 def test_cached_states_equal_recompute(gpu_device):
-    inp = make_inputs(1, 4, 1024, 128, 128, torch.float32, seed=6, state=True, state_std=1.0)
+    inp = make_inputs(1, 4, 1024, 128, 96, torch.float32, seed=6, state=True, state_std=1.0)
     s = O.slopes_baseline(4)
-    a = run_abi(inp, s, gpu_device, seg_len=256, cache=False)
-    c = run_abi(inp, s, gpu_device, seg_len=256, cache=True)
+    a = run_abi(inp, s, gpu_device, seg_len=256, cache=False, exact=True)
+    c = run_abi(inp, s, gpu_device, seg_len=256, cache=True, exact=True)
     for name in ("dq", "dk", "dv", "dkv_out"):
         assert torch.equal(a[name], c[name]), name
 
@@ -82,7 +88,7 @@ def test_segment_length_does_not_change_result(gpu_device):
     s = O.slopes_baseline(2)
     ref = oracle(inp, s)
     for seg in (64, 512, 2048):
-        check(run_abi(inp, s, gpu_device, seg_len=seg), ref, 1e-3, what=f"seg_len={seg}")
+        check(run_abi(inp, s, gpu_device, seg_len=seg, exact=True), ref, 1e-3, what=f"seg_len={seg}")
 
 
 def test_config0_fp32_full(gpu_device):
@@ -163,8 +169,8 @@ def test_narrow_bf16_heads_run_padded_on_mfma(gpu_device, d, e):
         check(got, oracle(inp, s), 2e-2, what=f"padded d={d} e={e} cache={cache}")
 
 
-@pytest.mark.parametrize("n,d,e", [(2047, 128, 128), (65, 128, 128), (700, 128, 64)])
-def test_ragged_bf16_length_is_split_head_mfma_tail_generic(gpu_device, n, d, e):
+@pytest.mark.parametrize("n,d,e", [(2047, 128, 128), (65, 128, 128), (700, 128, 64), (63, 128, 128), (1, 128, 128)])
+def test_ragged_bf16_length(gpu_device, n, d, e):
     inp = make_inputs(1, 3, n, d, e, torch.bfloat16, seed=n, state=True, state_std=1.0)
     s = O.slopes_alibi(3)
     ref = oracle(inp, s)
@@ -213,7 +219,23 @@ def test_mfma_fp32_special_slopes_and_padding(gpu_device):
     got = run_abi(inp, s, gpu_device, seg_len=128)
     assert all(torch.isfinite(v_).all() for v_ in got.values())
     check(got, oracle(inp, s), 1e-4, what="fp32 mfma s in {0, 1, 30}")
-    # narrow heads and a ragged length reach the same kernels through padding / splitting
+    # narrow heads (zero-padded) with a ragged length (masked last block)
     inp = make_inputs(1, 2, 300, 64, 96, torch.float32, seed=32, state=True, state_std=1.0)
     s = O.slopes_baseline(2)
     check(run_abi(inp, s, gpu_device), oracle(inp, s), 1e-4, what="fp32 narrow ragged")
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float16, 2e-2), (torch.float32, 1e-4)])
+@pytest.mark.parametrize("b,h,n,seg", [(1, 2, 100, 0), (2, 3, 333, 128), (1, 2, 1000, 256), (1, 1, 31, 0)])
+def test_mfma_ragged_lengths_in_kernel(gpu_device, dtype, tol, b, h, n, seg):
+    """A chunk length that is not a multiple of the block: the last block is masked inside the kernels."""
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(b, h, n, 128, 128, dtype) == _abi.PATH_MFMA
+    inp = make_inputs(b, h, n, 128, 128, dtype, seed=n + 3, state=True, state_std=1.0)
+    s = torch.tensor([0.3, 0.01, 2.0][:h])
+    ref = oracle(inp, s)
+    for cache in (False, True):
+        got = run_abi(inp, s, gpu_device, seg_len=seg, cache=cache)
+        assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
+        check(got, ref, tol, what=f"ragged {dtype} n={n} seg={seg} cache={cache}")
