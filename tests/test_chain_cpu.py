@@ -1,0 +1,127 @@
+"""Host logic of the operators without a GPU: the autograd Functions, the loopback state
+passing and the feature-slicing wrapper run here on CPU tensors with the two library calls
+(`_abi.chunk_fwd`, `_abi.chunk_bwd`) replaced by the oracle.  What is under test is the
+choreography around the calls -- zeroing KV, receive / clone / run / send, the reversed DKV
+chain, in-place state updates, slicing wide heads -- not the kernels."""
+import pytest
+import torch
+
+import lasp_amd
+from lasp_amd import _abi
+from oracle import lasp_oracle as O
+
+
+def _fake_fwd(q, k, v, s, kv_in=None, kv_out=None, seg_len=0):
+    o, kvo = O.ref_chunked_fwd(q, k, v, s, kv_in, 64, torch.float64)
+    if kv_out is not None:
+        kv_out.copy_(kvo.to(kv_out.dtype))
+    states = torch.zeros(1)  # stands for the segment-state cache
+    return o.to(q.dtype), states, 64
+
+
+def _fake_bwd(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len=0):
+    dq, dk, dv, dkvo = O.ref_chunked_bwd(q, k, v, s, do, kv_in, dkv_in, 64, torch.float64)
+    if dkv_out is not None:
+        dkv_out.copy_(dkvo.to(dkv_out.dtype))
+    return dq.to(q.dtype), dk.to(q.dtype), dv.to(q.dtype)
+
+
+@pytest.fixture(autouse=True)
+def _oracle_behind_the_abi(monkeypatch):
+    monkeypatch.setattr(_abi, "chunk_fwd", _fake_fwd)
+    monkeypatch.setattr(_abi, "chunk_bwd", _fake_bwd)
+    lasp_amd.destroy_parallel_groups()
+    yield
+    lasp_amd.destroy_parallel_groups()
+
+
+def _inputs(b, h, n, d, e, seed):
+    g = torch.Generator().manual_seed(seed)
+    q, k = [torch.randn(b, h, n, d, generator=g, dtype=torch.float64) for _ in range(2)]
+    v, do = [torch.randn(b, h, n, e, generator=g, dtype=torch.float64) for _ in range(2)]
+    return q, k, v, do
+
+
+def _chain(op_name, q, k, v, do, s, chunks):
+    op = getattr(lasp_amd, op_name)
+    b, h, n, d = q.shape
+    e = v.shape[-1]
+    step = n // chunks
+    lasp_amd.initialize_lasp(1, chunks)
+    KV = torch.full((b, h, d, e), 7.0, dtype=torch.float64)   # garbage on entry: the operator zeroes it
+    DKV = torch.full((b, h, d, e), -3.0, dtype=torch.float64)
+    outs, leaves, kv_after = [], [], []
+    for c in range(chunks):
+        lasp_amd.set_sequence_parallel_rank(c)
+        sl = slice(c * step, (c + 1) * step)
+        qc, kc, vc = [t[:, :, sl].clone().requires_grad_(True) for t in (q, k, v)]
+        if op_name == "lasp_naive":
+            o = op(qc, kc, vc, s)
+        elif op_name == "lasp_cache":
+            o = op(qc, kc, vc, s, torch.arange(step), KV, DKV)
+        else:
+            o = op(qc, kc, vc, s, KV, DKV)
+        outs.append(o)
+        leaves.append((qc, kc, vc))
+        kv_after.append(KV.clone())
+    for c in reversed(range(chunks)):
+        outs[c].backward(do[:, :, c * step:(c + 1) * step])
+    assert lasp_amd.loopback_pending() == []
+    cat = lambda i: torch.cat([l[i].grad for l in leaves], 2)
+    return torch.cat([o.detach() for o in outs], 2), cat(0), cat(1), cat(2), kv_after, DKV
+
+
+@pytest.mark.parametrize("op_name", ["lasp_fuse", "lasp_fuse_parallel", "lasp_cache", "lasp_naive"])
+def test_chain_choreography_equals_single_pass(op_name):
+    q, k, v, do = _inputs(2, 3, 256, 16, 8, seed=1)
+    s = O.slopes_alibi(3)
+    ref = O.ref_chunked(q, k, v, s, do, dtype=torch.float64)
+    o, dq, dk, dv, kv_after, DKV = _chain(op_name, q, k, v, do, s, chunks=4)
+    tol = 1e-6 if op_name == "lasp_naive" else 1e-12  # lasp_naive allocates its own float32 state buffers
+    for got, name in ((o, "o"), (dq, "dq"), (dk, "dk"), (dv, "dv")):
+        assert O.rel_err(got, ref[name]) < tol, (op_name, name)
+    if op_name != "lasp_naive":  # lasp_naive owns its buffers
+        # the caller's KV holds KV_out of the chunk just run; after the last chunk, of the whole sequence
+        assert O.rel_err(kv_after[-1], ref["kv_out"]) < 1e-12
+        _, kv1 = O.ref_chunked_fwd(q[:, :, :64], k[:, :, :64], v[:, :, :64], s, None, 64, torch.float64)
+        assert O.rel_err(kv_after[0], kv1) < 1e-12
+        # after the reversed chain the caller's DKV holds dL/dKV_in of the first chunk
+        assert O.rel_err(DKV, ref["dkv_out"]) < 1e-12
+
+
+def test_lightning_attn_and_wide_heads_are_sliced_and_summed():
+    # d = 320 -> feature slices [0,128) [128,256) [256,320): three calls whose outputs add up
+    q, k, v, do = _inputs(1, 2, 128, 320, 8, seed=2)
+    s = O.slopes_alibi(2)
+    ref = O.ref_chunked(q, k, v, s, do, dtype=torch.float64)
+    qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    o = lasp_amd.lightning_attn(qg, kg, vg, s)
+    o.backward(do)
+    assert O.rel_err(o, ref["o"]) < 1e-12
+    assert O.rel_err(qg.grad, ref["dq"]) < 1e-12
+    assert O.rel_err(kg.grad, ref["dk"]) < 1e-12
+    assert O.rel_err(vg.grad, ref["dv"]) < 1e-12
+
+
+def test_wide_heads_with_state_copy_back():
+    q, k, v, do = _inputs(1, 2, 128, 192, 8, seed=3)
+    s = O.slopes_alibi(2)
+    lasp_amd.initialize_lasp(1, 1)
+    KV = torch.empty(1, 2, 192, 8, dtype=torch.float64)
+    DKV = torch.empty_like(KV)
+    o = lasp_amd.lasp_fuse(q, k, v, s, KV, DKV)
+    ref_o, ref_kv = O.ref_chunked_fwd(q, k, v, s, None, 64, torch.float64)
+    assert O.rel_err(o, ref_o) < 1e-12
+    assert O.rel_err(KV, ref_kv) < 1e-12  # every feature slice of the state was written back
+
+
+def test_no_gradient_for_states_and_slopes():
+    q, k, v, do = _inputs(1, 2, 64, 8, 8, seed=4)
+    s = O.slopes_alibi(2).requires_grad_(True)
+    lasp_amd.initialize_lasp(1, 1)
+    KV = torch.zeros(1, 2, 8, 8, dtype=torch.float64)
+    DKV = torch.zeros_like(KV)
+    qg = q.clone().requires_grad_(True)
+    o = lasp_amd.lasp_fuse(qg, k, v, s, KV, DKV)
+    o.backward(do)
+    assert qg.grad is not None and s.grad is None
