@@ -212,7 +212,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
            const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
            const Geom &g, int item, char *smem) {
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
   const int c = lane & 31, hh = lane >> 5;
   const LoaderRole xr = x_role(tid), yr = yz_role(tid);
   const int chunk = tid & 15, rowq = tid >> 4;  // output copy role: 16-byte column, row
@@ -480,7 +481,8 @@ la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const f
              float *__restrict__ states, Geom g, int skip_seg) {
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
   const int c = lane & 31, hh = lane >> 5;
   const LoaderRole yr = yz_role(tid);
 

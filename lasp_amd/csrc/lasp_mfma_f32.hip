@@ -94,7 +94,8 @@ apply_body(const float *__restrict__ X, const float *__restrict__ Y, const float
            const float *__restrict__ S, const float *__restrict__ states, float *__restrict__ Out,
            const Geom &g, int item, char *smem) {
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
   const int c = lane & 31, hh = lane >> 5;
   const int cq = tid & 31, rq = tid >> 5;  // loader: 16-byte column, row (X) / group of four rows (Y, Z)
 
@@ -288,7 +289,8 @@ la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const f
                float *__restrict__ states, Geom g, int skip_seg) {
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {(w (.) Y)^T, Z^T}
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
   const int c = lane & 31, hh = lane >> 5;
   const int cq = tid & 31, rq = tid >> 5;
 
