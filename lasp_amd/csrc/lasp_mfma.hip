@@ -21,7 +21,7 @@
 // Work split inside a 256-thread workgroup (4 waves): wave w owns columns
 // [32w, 32w+32) of St and of the output, as four 32x32 fp32 MFMA accumulator
 // tiles that never leave registers; the 64x64 score tile is computed once,
-// cooperatively (one 32x32 quadrant per wave), masked, rounded to bf16 and shared
+// cooperatively (one 32x32 quadrant per wave), masked, rounded to 16 bits and shared
 // through LDS.  All products are arranged so that an accumulator tile can be fed
 // back as an MFMA operand without a shuffle: v_mfma_f32_32x32x16_bf16 leaves
 // C[8g+4hh+r][c] in register 4g+r of lane (c, hh) -- four consecutive rows per
@@ -36,14 +36,13 @@ namespace {
 // a register array to scratch memory)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef float float2_t __attribute__((ext_vector_type(2)));
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-// native vector types (HIP's u32x4 / u32x2 structs copy through memcpy, which can pin
-// a register array to scratch memory)
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
-typedef float float2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
+typedef uint16_t elem16_t;  // raw bits of one bf16 or fp16 element
 
 constexpr int F = 128;      // feature size (d = e)
 constexpr int BLK = 64;     // tokens per block
@@ -59,9 +58,6 @@ constexpr int OFF_SC = OFF_ZT + F * LDT;
 constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
 constexpr float LOG2E = 1.4426950408889634f;
 
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8;
-
 // Element policies: the kernels move 16-bit elements as raw bits and only touch their value
 // in three places -- widening one element, rounding two floats into a packed pair, and the
 // MFMA itself.
@@ -70,7 +66,7 @@ struct ElemBF16 {
     float2_t v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   }
-  // `bits` holds the element in its low (odd = false) or high (odd = true) half
+  // `word` holds the element in its low (odd = false) or high (odd = true) half
   static __device__ __forceinline__ float widen(uint32_t word, bool odd) {
     return __uint_as_float(odd ? (word & 0xffff0000u) : (word << 16));
   }
@@ -102,7 +98,7 @@ __device__ __forceinline__ float elem_f32(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
   return E::widen(w, x & 1);
 }
-__device__ __forceinline__ uint32_t bf_bits(const u32x4 &q, int x) {
+__device__ __forceinline__ uint32_t elem_bits(const u32x4 &q, int x) {
   const uint32_t w = (x >> 1) == 0 ? q.x : (x >> 1) == 1 ? q.y : (x >> 1) == 2 ? q.z : q.w;
   return (x & 1) ? (w >> 16) : (w & 0xffffu);
 }
@@ -164,8 +160,8 @@ __device__ __forceinline__ void store_transposed(char *tile, const u32x4 (&rows)
       out.x = E::pack(elem_f32<E>(rows[0], x) * w[0], elem_f32<E>(rows[1], x) * w[1]);
       out.y = E::pack(elem_f32<E>(rows[2], x) * w[2], elem_f32<E>(rows[3], x) * w[3]);
     } else {
-      out.x = bf_bits(rows[0], x) | (bf_bits(rows[1], x) << 16);
-      out.y = bf_bits(rows[2], x) | (bf_bits(rows[3], x) << 16);
+      out.x = elem_bits(rows[0], x) | (elem_bits(rows[1], x) << 16);
+      out.y = elem_bits(rows[2], x) | (elem_bits(rows[3], x) << 16);
     }
     *reinterpret_cast<u32x2 *>(tile + tr_off(f, role.rowq >> 1) + ((role.rowq & 1) << 3)) = out;
   }
@@ -208,8 +204,8 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 // partial; the aligned instantiation carries none of that bookkeeping.
 template <class E, bool REV, bool TRANS, bool RAGGED>
 __device__ __forceinline__ void
-apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
-           const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
+apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
+           const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
            const Geom &g, int item, char *smem) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -356,6 +352,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
       }
     }
     __builtin_amdgcn_s_setprio(0);
+    // (2) mask the quadrant with l^|a-b| (exponents <= 0 only), round it, share it through LDS;
+    //     scale the state term by the query decay
     if (q_active) {
       const int a = 32 * qI + c;
 #pragma unroll
@@ -441,8 +439,8 @@ apply_body(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf1
 
 template <class E, bool REV, bool TRANS, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
-la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z,
-         const float *__restrict__ S, const float *__restrict__ states, bf16_t *__restrict__ Out,
+la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
+         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
          Geom g) {
   extern __shared__ __align__(16) char smem[];
   apply_body<E, REV, TRANS, RAGGED>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
@@ -454,10 +452,10 @@ la_apply(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Y, const bf16_
 // XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
 template <class E, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
-la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t *__restrict__ V,
-        const bf16_t *__restrict__ DO, const float *__restrict__ S,
+la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+        const elem16_t *__restrict__ DO, const float *__restrict__ S,
         const float *__restrict__ kv_states, const float *__restrict__ dkv_states,
-        bf16_t *__restrict__ DQ, bf16_t *__restrict__ DK, bf16_t *__restrict__ DV, Geom g) {
+        elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
   extern __shared__ __align__(16) char smem[];
   const int n_items = g.b * g.h * g.n_seg;
   const int grp = blockIdx.x / 24, r = blockIdx.x - grp * 24;
@@ -477,7 +475,7 @@ la_bwd3(const bf16_t *__restrict__ Q, const bf16_t *__restrict__ K, const bf16_t
 // (b from the segment start, L its length), written token-free as 128 x 128 fp32.
 template <class E, bool REV, bool RAGGED>
 __global__ void __launch_bounds__(NTHR, 2)
-la_seg_state(const bf16_t *__restrict__ Y, const bf16_t *__restrict__ Z, const float *__restrict__ S,
+la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
   const int tid = threadIdx.x;
@@ -594,9 +592,9 @@ int launch_apply(const void *x, const void *y, const void *z, const float *s, co
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply<E, REV, TRANS, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)x, (const bf16_t *)y,
-                                                                 (const bf16_t *)z, s, states,
-                                                                 (bf16_t *)out, g);
+  la_apply<E, REV, TRANS, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
+                                                                 (const elem16_t *)z, s, states,
+                                                                 (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
@@ -608,10 +606,10 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3<E, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const bf16_t *)a.q, (const bf16_t *)a.k,
-                                                    (const bf16_t *)a.v, (const bf16_t *)a.d_o, a.s,
-                                                    kv_states, dkv_states, (bf16_t *)a.dq,
-                                                    (bf16_t *)a.dk, (bf16_t *)a.dv, g);
+  la_bwd3<E, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                    (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
+                                                    kv_states, dkv_states, (elem16_t *)a.dq,
+                                                    (elem16_t *)a.dk, (elem16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
@@ -623,7 +621,7 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, RAGGED><<<grid, NTHR, 0, st>>>((const bf16_t *)y, (const bf16_t *)z, s, states, g,
+  la_seg_state<E, REV, RAGGED><<<grid, NTHR, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
                                                       skip_seg);
   return (int)hipGetLastError();
 }
