@@ -34,8 +34,8 @@ BYTES_BWD_PER_TH = 1792        # read Q,K,V,dO + write dQ,dK,dV
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
 # (profiles/pmc_hbm_bytes_config2.txt); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0, the
 # factors a plain 1 GiB device copy shows for the same counters.
-TRAFFIC_BWD3_BYTES = 2709071 * 1024   # 2 x 961 319 KiB fetched + 786 432 KiB written
-TRAFFIC_APPLY_BYTES = 1081505 * 1024  # 2 x 409 681 KiB fetched + 262 144 KiB written
+TRAFFIC_BWD3_BYTES = 2708338 * 1024   # 2 x 960 953 KiB fetched + 786 432 KiB written
+TRAFFIC_APPLY_BYTES = 1081509 * 1024  # 2 x 409 683 KiB fetched + 262 144 KiB written
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
