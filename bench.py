@@ -8,9 +8,9 @@ public operator (lightning_attn + autograd) on the headline workload (TNL-1B hea
 b=1, h=16, n=65536, d=e=128, bf16, Q/K/V/dO ~ N(0,1)/sqrt(d), slopes
 2^(-8(i+1)/16); inputs are resident in HBM before the timed region.
 Prints ONE JSON line (metric = fwd+bwd tokens/s) that also carries
-  roofline     -- la_apply, the dominant kernel, against the HBM roof: algorithmic
+  roofline     -- la_bwd3, the dominant kernel, against the HBM roof: algorithmic
                   bytes per launch / its mean launch duration (HIP events around
-                  every launch, on the launch stream)
+                  every launch, on the launch stream); roofline_fwd: the same for la_apply
   cpu_baseline -- the CPU oracle (fp32 torch port of the same recurrence) timed on
                   the host cores on one pass of the same workload.
 """
