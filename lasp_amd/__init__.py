@@ -2,6 +2,7 @@
 
 Public names follow the reference package (lasp/__init__.py:1-6).
 """
+from .lasp_cache import *  # noqa: F401,F403
 from .lasp_fuse import *  # noqa: F401,F403
 from .lasp_fuse_parallel import *  # noqa: F401,F403
 from .lasp_naive import *  # noqa: F401,F403

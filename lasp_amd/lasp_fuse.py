@@ -1,9 +1,29 @@
 """lasp_fuse: per-rank chunk with KV in/out, states recomputed in backward (lasp/lasp_fuse.py)."""
 import torch
 
+from . import _abi
 from ._chain import ChunkFunction, run_sliced
 
 __all__ = ["LaspFuse", "lasp_fuse_", "lasp_fuse"]
+
+
+def lasp_forward(q, k, v, s, KV):
+    """Launch shim with the signature of lasp/lasp_fuse.py:356-406.
+
+    Returns o for one chunk.  KV, float32 (b, h, d, e), holds the incoming state and
+    is overwritten with the outgoing one, as the reference kernel does (:126-127).
+    """
+    o, _, _ = _abi.chunk_fwd(q, k, v, s, kv_in=KV, kv_out=KV)
+    return o
+
+
+def lasp_backward(q, k, v, s, do, KV, DKV):
+    """Launch shim with the signature of lasp/lasp_fuse.py:409-475.
+
+    KV is the state that entered the forward (the copy saved at :496); DKV holds the
+    incoming dKV and is overwritten with the outgoing one.  Returns (dq, dk, dv).
+    """
+    return _abi.chunk_bwd(q, k, v, s, do, kv_in=KV, dkv_in=DKV, dkv_out=DKV)
 
 
 class LaspFuse(torch.autograd.Function):

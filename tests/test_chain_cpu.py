@@ -125,3 +125,41 @@ def test_no_gradient_for_states_and_slopes():
     o = lasp_amd.lasp_fuse(qg, k, v, s, KV, DKV)
     o.backward(do)
     assert qg.grad is not None and s.grad is None
+
+
+def test_launch_shims_keep_the_reference_signatures_and_aliasing():
+    """lasp_fuse.lasp_forward / lasp_backward update KV / DKV in place; the lasp_fuse_parallel
+    pair returns new state tensors and leaves the caller's buffers alone
+    (lasp/lasp_fuse.py:356-475, lasp/lasp_fuse_parallel.py:833-1070)."""
+    import importlib
+
+    # the package attributes of these names are the operators (as in the reference), so go through sys.modules
+    LF = importlib.import_module("lasp_amd.lasp_fuse")
+    LP = importlib.import_module("lasp_amd.lasp_fuse_parallel")
+
+    q, k, v, do = _inputs(1, 2, 128, 16, 8, seed=5)
+    s = O.slopes_alibi(2)
+    g = torch.Generator().manual_seed(6)
+    kv0 = torch.randn(1, 2, 16, 8, generator=g, dtype=torch.float64)
+    dkv0 = torch.randn(1, 2, 16, 8, generator=g, dtype=torch.float64)
+    ref = O.ref_chunked(q, k, v, s, do, kv0, dkv0, dtype=torch.float64)
+
+    KV, DKV = kv0.clone(), dkv0.clone()
+    o = LF.lasp_forward(q, k, v, s, KV)
+    assert O.rel_err(o, ref["o"]) < 1e-12 and O.rel_err(KV, ref["kv_out"]) < 1e-12
+    dq, dk, dv = LF.lasp_backward(q, k, v, s, do, kv0, DKV)
+    assert max(O.rel_err(dq, ref["dq"]), O.rel_err(dk, ref["dk"]), O.rel_err(dv, ref["dv"])) < 1e-12
+    assert O.rel_err(DKV, ref["dkv_out"]) < 1e-12
+
+    KV, DKV = kv0.clone(), dkv0.clone()
+    o, cache, KV_out = LP.lasp_forward(q, k, v, s, KV, 128, 64)
+    assert torch.equal(KV, kv0) and O.rel_err(KV_out, ref["kv_out"]) < 1e-12 and O.rel_err(o, ref["o"]) < 1e-12
+    dq, dk, dv, DKV_out = LP.lasp_backward(q, k, v, s, do, cache, kv0, DKV, 128, 64)
+    assert torch.equal(DKV, dkv0) and O.rel_err(DKV_out, ref["dkv_out"]) < 1e-12
+    assert max(O.rel_err(dq, ref["dq"]), O.rel_err(dk, ref["dk"]), O.rel_err(dv, ref["dv"])) < 1e-12
+
+
+def test_lasp_cache_module_path():
+    from lasp_amd.lasp_cache import LaspCache, lasp_cache  # noqa: F401
+
+    assert lasp_cache is lasp_amd.lasp_cache and callable(lasp_amd.lasp_cache)

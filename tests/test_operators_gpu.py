@@ -170,3 +170,35 @@ def test_graph_capture_replays_match_eager(gpu_device):
             assert torch.equal(a, e)
     ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s.cpu(), inp["do"], dtype=torch.float64)
     assert O.rel_err(torch.cat(captured[:chunks], 2), ref["o"]) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype,e", [(torch.bfloat16, 128), (torch.float32, 128), (torch.bfloat16, 64)])
+def test_launch_shims_against_oracle(gpu_device, dtype, e):
+    """lasp_fuse.lasp_forward/lasp_backward (states in place) and the lasp_fuse_parallel pair
+    (new state tensors, segment-state cache handed from forward to backward) on one chunk with
+    incoming KV and dKV (lasp/lasp_fuse.py:356-475, lasp/lasp_fuse_parallel.py:833-1070)."""
+    import importlib
+
+    from tests.helpers import TOL, check, oracle
+
+    LF = importlib.import_module("lasp_amd.lasp_fuse")
+    LP = importlib.import_module("lasp_amd.lasp_fuse_parallel")
+    dev = gpu_device
+    b, h, n, d = 1, 4, 1024, 128
+    s = O.slopes_baseline(h)
+    inp = make_inputs(b, h, n, d, e, dtype, seed=31, scale=d ** -0.5, state=True, device=dev)
+    ref = oracle(inp, s)
+    q, k, v, do, sd = inp["q"], inp["k"], inp["v"], inp["do"], s.to(dev)
+
+    KV, DKV = inp["kv"].clone(), inp["dkv"].clone()
+    o = LF.lasp_forward(q, k, v, sd, KV)
+    dq, dk, dv = LF.lasp_backward(q, k, v, sd, do, inp["kv"], DKV)
+    torch.cuda.synchronize()
+    check(dict(o=o, kv_out=KV, dq=dq, dk=dk, dv=dv, dkv_out=DKV), ref, TOL[dtype], what="lasp_fuse shims")
+
+    KV, DKV = inp["kv"].clone(), inp["dkv"].clone()
+    o, cache, KV_out = LP.lasp_forward(q, k, v, sd, KV, 256, 64)
+    dq, dk, dv, DKV_out = LP.lasp_backward(q, k, v, sd, do, cache, KV, DKV, 256, 64)
+    torch.cuda.synchronize()
+    assert torch.equal(KV, inp["kv"]) and torch.equal(DKV, inp["dkv"])
+    check(dict(o=o, kv_out=KV_out, dq=dq, dk=dk, dv=dv, dkv_out=DKV_out), ref, TOL[dtype], what="lasp_fuse_parallel shims")
