@@ -239,3 +239,25 @@ def test_mfma_ragged_lengths_in_kernel(gpu_device, dtype, tol, b, h, n, seg):
         got = run_abi(inp, s, gpu_device, seg_len=seg, cache=cache)
         assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
         check(got, ref, tol, what=f"ragged {dtype} n={n} seg={seg} cache={cache}")
+
+
+def test_seeded_random_shapes(gpu_device):
+    """24 shapes drawn from a fixed seed: any n (ragged against blocks and against segments), narrow and
+    full heads, the three dtypes, forced and planned segment lengths, with and without incoming states."""
+    import random
+
+    rng = random.Random(20240607)
+    dtypes = [torch.bfloat16, torch.float16, torch.float32]
+    for case in range(24):
+        b, h = rng.choice([1, 2]), rng.randint(1, 5)
+        n = rng.choice([rng.randint(1, 130), rng.randint(131, 1500)])
+        d, e = rng.choice([128, 128, 64, 48]), rng.choice([128, 128, 64, 16])
+        dtype = rng.choice(dtypes)
+        seg = rng.choice([0, 0, 64, 128, 256, 512])
+        state = rng.random() < 0.6
+        s = rng.choice([O.slopes_baseline(h), O.slopes_alibi(h), torch.zeros(h, 1, 1)])
+        inp = make_inputs(b, h, n, d, e, dtype, seed=1000 + case, scale=0.3, state=state, state_std=0.5)
+        what = f"case {case}: b={b} h={h} n={n} d={d} e={e} {dtype} seg={seg} state={state}"
+        print(what, flush=True)
+        got = run_abi(inp, s, gpu_device, seg_len=seg, cache=bool(case & 1))
+        check(got, oracle(inp, s), 1e-4 if dtype == torch.float32 else 2e-2, what=what)
