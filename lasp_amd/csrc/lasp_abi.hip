@@ -127,6 +127,13 @@ int lasp_profile_begin(int max_launches) {
   for (int i = 0; i < max_launches; ++i) {
     hipError_t e1 = hipEventCreate(&p[i].start), e2 = hipEventCreate(&p[i].stop);
     if (e1 != hipSuccess || e2 != hipSuccess) {
+      if (e1 == hipSuccess) (void)hipEventDestroy(p[i].start);
+      if (e2 == hipSuccess) (void)hipEventDestroy(p[i].stop);
+      for (int j = 0; j < i; ++j) {
+        (void)hipEventDestroy(p[j].start);
+        (void)hipEventDestroy(p[j].stop);
+      }
+      delete[] p;
       set_error("lasp_profile_begin: hipEventCreate failed");
       return (int)(e1 != hipSuccess ? e1 : e2);
     }
