@@ -57,6 +57,11 @@ def test_config2_headline_shape(gpu_device):
     torch.cuda.synchronize()
     heads = [0, 7, 15]
     _check_heads(got, _oracle_heads(q, k, v, do, s, heads), heads, ("o", "dq", "dk", "dv"))
+    # no atomics, fixed reduction order: a second run gives the same bits
+    again = _fwd_bwd(q, k, v, do, s)
+    for name in ("o", "dq", "dk", "dv"):
+        assert torch.equal(again[name], got[name]), name
+    del again
     # chunk chain (4 x 16384, states carried) == single pass
     kv = torch.zeros(b, h, d, d, device=dev)
     outs = []
