@@ -41,6 +41,8 @@ constexpr int kMaxFeature = 128;     // d and e of one launch (the Python wrappe
 constexpr int kSegQuantum = 64;      // segment lengths are multiples of this
 constexpr int64_t kTargetGroups = 512;  // workgroups wanted per launch (2 per CU on 256 CUs)
 constexpr int kMinSeg = 256;
+constexpr int kPreferredSeg = 1024;     // preferred lower bound while kMinGroups workgroups remain
+constexpr int64_t kMinGroups = 256;     // one workgroup per CU
 
 int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
   if (dtype != LASP_DTYPE_F32 && dtype != LASP_DTYPE_BF16 && dtype != LASP_DTYPE_F16) {
@@ -65,6 +67,11 @@ int default_seg_len(int b, int h, int64_t n) {
   int64_t len = n / (want > 0 ? want : 1);
   len = (len / kMinSeg) * kMinSeg;
   if (len < kMinSeg) len = kMinSeg;
+  // Segments shorter than kPreferredSeg spend a visible share of their time on the 64 KiB
+  // state each one loads and the scan has to carry; one workgroup per CU of longer
+  // segments measured faster than two of shorter ones.
+  if (len < kPreferredSeg && bh * ((n + kPreferredSeg - 1) / kPreferredSeg) >= kMinGroups)
+    len = kPreferredSeg;
   return (int)len;
 }
 
