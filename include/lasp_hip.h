@@ -55,7 +55,9 @@ extern "C" {
 
 /* Which kernel family a shape/dtype is served by (lasp_kernel_path). */
 #define LASP_PATH_GENERIC 0 /* fp32-FMA kernels: any dtype, any n, d,e <= 128 */
-#define LASP_PATH_MFMA 1    /* MFMA kernels: d = e = 128, any dtype, any n (a ragged tail is masked) */
+#define LASP_PATH_MFMA 1    /* MFMA kernels, any n (a ragged tail is masked): bf16 / fp16 with d and e
+                               multiples of 8 (rows narrower than 128 are read zero-extended), fp32 with
+                               d = e = 128 */
 
 int lasp_abi_version(void);
 
@@ -69,7 +71,8 @@ const char *lasp_last_error(void);
  * lasp_plan returns the default seg_len for a shape (pass it, or any other
  * positive multiple of 64, to the calls below); n_seg = ceil(n / seg_len) and
  * the byte size of ONE segment-state array are written through the pointers
- * (either may be NULL).  Replaces the BLOCK/NUM_BLOCK choice of
+ * (either may be NULL).  The array is opaque: the MFMA kernels keep every state
+ * zero-extended to 128 x 128 floats, the generic ones as d x e.  Replaces the BLOCK/NUM_BLOCK choice of
  * lasp/lasp_fuse_parallel.py:1080-1085 and the `kv` buffer shape of :876.
  */
 int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0,

@@ -166,12 +166,13 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     s = _slopes(s, h, dev)
     _check_state("kv_in", kv_in, b, h, d, e)
     _check_state("kv_out", kv_out, b, h, d, e)
-    seg_len, n_seg, _ = plan(b, h, n, d, e, q.dtype, seg_len)
+    seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
     with torch.cuda.device(dev):
         o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
         states = None
         if n_seg > 1 or kv_in is not None or kv_out is not None:
-            states = torch.empty((b, h, n_seg, d, e), dtype=torch.float32, device=dev)
+            # the library decides how a state is stored (d x e, or zero-extended to 128 x 128)
+            states = torch.empty((b, h, n_seg, state_bytes // (4 * b * h * n_seg)), dtype=torch.float32, device=dev)
         rc = lib.lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
                                 o.data_ptr(), _ptr(states), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
                                 torch.cuda.current_stream(dev).cuda_stream)
@@ -194,10 +195,11 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
     _check_state("dkv_out", dkv_out, b, h, d, e)
     seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
     if kv_seg_states is not None:
-        if (kv_seg_states.dtype != torch.float32 or tuple(kv_seg_states.shape) != (b, h, n_seg, d, e)
+        if (kv_seg_states.dtype != torch.float32 or kv_seg_states.numel() * 4 != state_bytes
                 or not kv_seg_states.is_contiguous()):
-            raise LaspError(f"kv_seg_states must be contiguous float32 {(b, h, n_seg, d, e)}, got "
-                            f"{kv_seg_states.dtype} {tuple(kv_seg_states.shape)}")
+            raise LaspError(f"kv_seg_states must be the contiguous float32 array of {state_bytes} bytes that "
+                            f"chunk_fwd returned for this shape, got {kv_seg_states.dtype} "
+                            f"{tuple(kv_seg_states.shape)}")
     with torch.cuda.device(dev):
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
@@ -214,17 +216,20 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
 
 
 # ---------------------------------------------------------------------------------------
-# Narrow heads on the MFMA kernels.  The MFMA kernels take d = e = 128 only.  A call with
-# narrower features (the reference's own test uses e = 64, tests/test.py:95) is zero-padded
-# to 128 here: zero feature columns add nothing to q.k, to the outputs or to the states, so the
-# results are exact, and the call runs an order of magnitude faster than on the generic
-# fp32-FMA kernels.  Everything else goes to the library unchanged.
+# Narrow heads on the MFMA kernels.  The 16-bit MFMA kernels read rows of d, e <= 128 features
+# zero-extended when d and e are multiples of 8 (the reference's own test uses e = 64,
+# tests/test.py:95); the fp32 MFMA kernels take d = e = 128 only.  Any other narrow shape is
+# zero-padded to 128 here: zero feature columns add nothing to q.k, to the outputs or to the
+# states, so the results are exact, and the call runs an order of magnitude faster than on
+# the generic fp32-FMA kernels.  Everything else goes to the library unchanged.
 _MFMA_F = 128
 
 
 def _pad_to_mfma(q, v) -> bool:
     d, e = q.shape[3], v.shape[3]
-    return q.dtype in DTYPE_CODE and d <= _MFMA_F and e <= _MFMA_F and (d < _MFMA_F or e < _MFMA_F)
+    if q.dtype not in DTYPE_CODE or d > _MFMA_F or e > _MFMA_F or (d == _MFMA_F and e == _MFMA_F):
+        return False
+    return q.dtype == torch.float32 or d % 8 != 0 or e % 8 != 0
 
 
 def _pad_last(t, size):

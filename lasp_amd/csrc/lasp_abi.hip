@@ -43,6 +43,7 @@ constexpr int64_t kTargetGroups = 512;  // workgroups wanted per launch (2 per C
 constexpr int kMinSeg = 256;
 constexpr int kPreferredSeg = 1024;     // preferred lower bound while kMinGroups workgroups remain
 constexpr int64_t kMinGroups = 256;     // one workgroup per CU
+constexpr int64_t kMaxSeg = 1 << 24;    // offsets inside a segment stay within 32 bits
 
 int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
   if (dtype != LASP_DTYPE_F32 && dtype != LASP_DTYPE_BF16 && dtype != LASP_DTYPE_F16) {
@@ -64,15 +65,26 @@ int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
 int default_seg_len(int b, int h, int64_t n) {
   const int64_t bh = (int64_t)b * h;
   const int64_t want = (kTargetGroups + bh - 1) / bh;  // segments per (b, h)
-  int64_t len = n / (want > 0 ? want : 1);
-  len = (len / kMinSeg) * kMinSeg;
-  if (len < kMinSeg) len = kMinSeg;
+  // rounded up, so that no more than `want` segments result: one workgroup more than the chip
+  // holds at once would cost a second pass over the CUs
+  int64_t len = (n + want - 1) / want;
+  len = ((len + kMinSeg - 1) / kMinSeg) * kMinSeg;
   // Segments shorter than kPreferredSeg spend a visible share of their time on the 64 KiB
   // state each one loads and the scan has to carry; one workgroup per CU of longer
   // segments measured faster than two of shorter ones.
   if (len < kPreferredSeg && bh * ((n + kPreferredSeg - 1) / kPreferredSeg) >= kMinGroups)
     len = kPreferredSeg;
+  if (len > kMaxSeg) len = kMaxSeg;
   return (int)len;
+}
+
+// The 16-bit MFMA kernels work on 128 features and read narrower rows zero-extended; their
+// 8-byte loads and 16-byte stores need every row to start on such a boundary.
+bool mfma_eligible(int d, int e, int dtype) {
+  return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && d % 8 == 0 && e % 8 == 0;
+}
+bool mfma_f32_eligible(int d, int e, int dtype) {
+  return dtype == LASP_DTYPE_F32 && d == kMaxFeature && e == kMaxFeature;
 }
 
 int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
@@ -96,18 +108,14 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   g->e = e;
   g->seg_len = seg_len;
   g->n_seg = (int)n_seg;
+  const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
+  g->sd = padded_states ? kMaxFeature : d;
+  g->se = padded_states ? kMaxFeature : e;
   return 0;
 }
 
-bool mfma_eligible(const Geom &g, int dtype) {
-  return (dtype == LASP_DTYPE_BF16 || dtype == LASP_DTYPE_F16) && g.d == 128 && g.e == 128;
-}
-bool mfma_f32_eligible(const Geom &g, int dtype) {
-  return dtype == LASP_DTYPE_F32 && g.d == 128 && g.e == 128;
-}
-
 size_t state_bytes_of(const Geom &g) {
-  return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.d * g.e;
+  return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.sd * g.se;
 }
 
 }  // namespace
@@ -196,7 +204,7 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
   Geom g;
   int rc = make_geom(b, h, n, d, e, dtype, 0, &g);
   if (rc) return rc;
-  return (mfma_eligible(g, dtype) || mfma_f32_eligible(g, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
+  return (mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
 }
 
 int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, const float *kv_in,
@@ -216,9 +224,9 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
   }
   FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype)       ? mfma_fwd(a, g, dtype, st)
-       : mfma_f32_eligible(g, dtype) ? mfma_f32_fwd(a, g, st)
-                                     : generic_fwd(a, g, dtype, st);
+  rc = mfma_eligible(d, e, dtype)       ? mfma_fwd(a, g, dtype, st)
+       : mfma_f32_eligible(d, e, dtype) ? mfma_f32_fwd(a, g, st)
+                                        : generic_fwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_fwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }
@@ -255,9 +263,9 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
   }
   if (need_kv) a.ws_kv = wp;
   hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(g, dtype)       ? mfma_bwd(a, g, dtype, st)
-       : mfma_f32_eligible(g, dtype) ? mfma_f32_bwd(a, g, st)
-                                     : generic_bwd(a, g, dtype, st);
+  rc = mfma_eligible(d, e, dtype)       ? mfma_bwd(a, g, dtype, st)
+       : mfma_f32_eligible(d, e, dtype) ? mfma_f32_bwd(a, g, st)
+                                        : generic_bwd(a, g, dtype, st);
   if (rc > 0) set_error("lasp_chunk_bwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }

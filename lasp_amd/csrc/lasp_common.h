@@ -55,6 +55,8 @@ struct Geom {
   int d, e;     // feature sizes of q/k and v/o
   int seg_len;  // tokens per segment (multiple of 64)
   int n_seg;    // ceil(n / seg_len)
+  int sd, se;   // rows and columns of one segment state as stored in the workspace: d x e for the
+                // generic kernels, 128 x 128 (zero beyond d, e) for the MFMA kernels
 };
 
 // Host-side launchers (each returns a hipError_t as int, or a negative LASP_E_*).

@@ -321,15 +321,19 @@ generic_bwd_dkdv(const T *__restrict__ Q, const T *__restrict__ K, const T *__re
 __global__ void __launch_bounds__(256)
 segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *carry_out,
                     const float *__restrict__ S, Geom g, int reverse) {
-  const int64_t de = (int64_t)g.d * g.e;
+  // one thread per element of the stored (sd x se) state; the carries are d x e
+  const int64_t sde = (int64_t)g.sd * g.se;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t total = (int64_t)g.b * g.h * de;
+  const int64_t total = (int64_t)g.b * g.h * sde;
   if (idx >= total) return;
-  const int bh = (int)(idx / de);
-  const int64_t el = idx - (int64_t)bh * de;
+  const int bh = (int)(idx / sde);
+  const int64_t el = idx - (int64_t)bh * sde;
+  const int row = (int)(el / g.se), col = (int)(el - (int64_t)row * g.se);
+  const bool in_carry = row < g.d && col < g.e;  // the padding of a stored state stays zero
+  const int64_t cidx = ((int64_t)bh * g.d + row) * g.e + col;
   const float s = S[bh % g.h];
-  float run = carry_in ? carry_in[idx] : 0.f;
-  float *p = states + (int64_t)bh * g.n_seg * de + el;
+  float run = (carry_in && in_carry) ? carry_in[cidx] : 0.f;
+  float *p = states + (int64_t)bh * g.n_seg * sde + el;
   const float full = expf(-s * (float)g.seg_len);
   const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
   const float tail = expf(-s * (float)last_len);
@@ -342,19 +346,19 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
     for (int u = 0; u < BATCH; ++u) {
       const int k = done + u;
       const int sg = reverse ? g.n_seg - 1 - k : k;
-      local[u] = k < g.n_seg ? p[(int64_t)sg * de] : 0.f;
+      local[u] = k < g.n_seg ? p[(int64_t)sg * sde] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < BATCH; ++u) {
       const int k = done + u;
       if (k < g.n_seg) {
         const int sg = reverse ? g.n_seg - 1 - k : k;
-        p[(int64_t)sg * de] = run;
+        p[(int64_t)sg * sde] = run;
         run = fmaf(sg == g.n_seg - 1 ? tail : full, run, local[u]);
       }
     }
   }
-  if (carry_out) carry_out[idx] = run;
+  if (carry_out && in_carry) carry_out[cidx] = run;
 }
 
 template <class K>
@@ -435,7 +439,7 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
 
 int launch_segment_scan(float *states, const float *carry_in, float *carry_out, const float *s,
                         const Geom &g, int reverse, hipStream_t st) {
-  const int64_t total = (int64_t)g.b * g.h * g.d * g.e;
+  const int64_t total = (int64_t)g.b * g.h * g.sd * g.se;
   const unsigned grid = (unsigned)((total + 255) / 256);
   ProfScope prof(KC_SCAN, st);
   segment_scan_kernel<<<grid, 256, 0, st>>>(states, carry_in, carry_out, s, g, reverse);

@@ -1,5 +1,7 @@
-// bf16 / fp16 MFMA kernels for d = e = 128 (gfx950, wave64); a chunk length that is not a
-// multiple of 64 ends in one partial block (RAGGED instantiations).
+// bf16 / fp16 MFMA kernels (gfx950, wave64).  The arithmetic is laid out for d = e = 128.
+// Three instantiations of every kernel: M_ALIGNED (chunk length a multiple of 64), M_RAGGED
+// (one partial last block) and M_NARROW (rows of d, e < 128 features, multiples of 8, read
+// zero-extended to 128 and written back at their own width; any chunk length).
 //
 // One kernel, `la_apply`, evaluates a causal (or anti-causal) decayed linear
 // attention over a segment of 64-token blocks given the state entering it:
@@ -57,6 +59,7 @@ constexpr int OFF_ZT = OFF_YT + F * LDT;
 constexpr int OFF_SC = OFF_ZT + F * LDT;
 constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
 constexpr float LOG2E = 1.4426950408889634f;
+enum Mode { M_ALIGNED = 0, M_RAGGED = 1, M_NARROW = 2 };
 
 // Element policies: the kernels move 16-bit elements as raw bits and only touch their value
 // in three places -- widening one element, rounding two floats into a packed pair, and the
@@ -179,6 +182,36 @@ __device__ __forceinline__ u32x4 load_row_pieces(const u32x2 *row, const LoaderR
   return r;
 }
 
+// Narrow or partial tiles: a thread's two pieces of the row that starts `row_bytes` (uniform
+// across the workgroup) past `tile`, at the thread's own byte offset `lane_off` (32 bits,
+// loop-invariant); a piece that lies beyond the row width, or the whole row, reads as zeros.
+struct PieceMask {
+  bool lo, hi;
+};
+__device__ __forceinline__ u32x4 load_row_pieces(const char *tile, int64_t row_bytes, uint32_t lane_off,
+                                                 PieceMask ok, bool row_ok) {
+  const char *p = tile + row_bytes;
+  const u32x2 zero = {0u, 0u};
+  const u32x2 lo = (row_ok && ok.lo) ? *reinterpret_cast<const u32x2 *>(p + lane_off) : zero;
+  const u32x2 hi = (row_ok && ok.hi) ? *reinterpret_cast<const u32x2 *>(p + lane_off + 16) : zero;
+  u32x4 r;
+  r.x = lo.x;
+  r.y = lo.y;
+  r.z = hi.x;
+  r.w = hi.y;
+  return r;
+}
+// thread-own part of the address: `row` rows down, then the thread's first piece
+__device__ __forceinline__ uint32_t lane_offset(const LoaderRole &role, int row, int units) {
+  return (uint32_t)((row * units + 4 * role.G + role.j) * 8);
+}
+__device__ __forceinline__ PieceMask piece_mask(const LoaderRole &role, int units) {
+  PieceMask m;
+  m.lo = 4 * role.G + role.j < units;
+  m.hi = 4 * role.G + 2 + role.j < units;
+  return m;
+}
+
 struct SegWork {
   int bh, seg;
   int64_t tok0;  // first token of the segment
@@ -200,13 +233,17 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 }
 
 // ------------------------------------------------------------------------------
-// RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
-// partial; the aligned instantiation carries none of that bookkeeping.
-template <class E, bool REV, bool TRANS, bool RAGGED>
+// M_RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
+// partial.  M_NARROW: in addition X and Y rows hold `fa` features, Z and Out rows `fb`
+// (multiples of 8, at most 128); feature steps, state tiles and waves that would only see the
+// zero extension are skipped.  M_ALIGNED carries none of that bookkeeping; fa and fb are read
+// in M_NARROW only.
+template <class E, bool REV, bool TRANS, int MODE>
 __device__ __forceinline__ void
 apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
-           const Geom &g, int item, char *smem) {
+           const Geom &g, int fa, int fb, int item, char *smem) {
+  constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
@@ -216,11 +253,14 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 
   const SegWork sw = seg_work(g, item);
   const float sl = S[sw.bh % g.h] * LOG2E;
-  const int64_t base = ((int64_t)sw.bh * g.n + sw.tok0) * F;
-  const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + base);
-  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + base);
-  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + base);
-  u32x4 *Og = reinterpret_cast<u32x4 *>(Out + base);
+  const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;  // first row of the segment
+  const int xw = NARROW ? fa : F, zw = NARROW ? fb : F;  // row widths in elements
+  const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + row0 * xw);
+  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * xw);
+  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * zw);
+  u32x4 *Og = reinterpret_cast<u32x4 *>(Out + row0 * zw);
+  const int xu = xw / 4, zu = zw / 4;  // 8-byte units per row
+  const int ou = zw / 8;               // 16-byte units per output row
 
   // ---- constants (all exponents <= 0)
   const float blockdec = decay(sl, (float)BLK);
@@ -236,6 +276,9 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
     const int b = 4 * yr.rowq + r;
     kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
   }
+  // M_NARROW: a wave whose 32 output columns all lie past the width of Z has only its share of
+  // the score tile to compute
+  const bool wave_active = !NARROW || 32 * w < fb;
   const int qI = w >> 1, qJ = w & 1;  // score quadrant of this wave: queries 32*qI.., keys 32*qJ..
   const bool q_active = REV ? !(qI == 1 && qJ == 0) : !(qI == 0 && qJ == 1);
 
@@ -260,30 +303,48 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 
   // ---- block loader: registers <- global, LDS <- registers
   u32x4 nx[4], ny[4], nz[4];
+  // M_NARROW addressing: uniform tile and row offsets plus these per-thread constants
+  const uint32_t x_off = lane_offset(xr, xr.rowq, xu), y_off = lane_offset(yr, 4 * yr.rowq, xu),
+                 z_off = lane_offset(yr, 4 * yr.rowq, zu);
+  const PieceMask x_ok = piece_mask(xr, xu), y_ok = piece_mask(yr, xu), z_ok = piece_mask(yr, zu);
   // a partial block (the end of a ragged chunk) reads its missing rows as zeros
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
-    const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units (32 per row)
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    if (!RAGGED || len == BLK) {
+    if (!NARROW) {
+      const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units (32 per row)
+      if (!RAGGED || len == BLK) {
 #pragma unroll
-      for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
+        for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
-        nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
+        for (int r = 0; r < 4; ++r) {
+          ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
+          nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
+        }
+      } else {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int row = xr.rowq + 16 * it;
+          nx[it] = row < len ? load_row_pieces(Xg + off + row * 32, xr) : zero;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = 4 * yr.rowq + r;
+          ny[r] = row < len ? load_row_pieces(Yg + off + row * 32, yr) : zero;
+          nz[r] = row < len ? load_row_pieces(Zg + off + row * 32, yr) : zero;
+        }
       }
     } else {
-      const u32x4 zero = {0u, 0u, 0u, 0u};
+      const int64_t xblk = (int64_t)blk * BLK * xu * 8, zblk = (int64_t)blk * BLK * zu * 8;  // bytes
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int row = xr.rowq + 16 * it;
-        nx[it] = row < len ? load_row_pieces(Xg + off + row * 32, xr) : zero;
-      }
+      for (int it = 0; it < 4; ++it)
+        nx[it] = load_row_pieces(reinterpret_cast<const char *>(Xg), xblk + (int64_t)(16 * it) * xu * 8, x_off,
+                                 x_ok, xr.rowq + 16 * it < len);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int row = 4 * yr.rowq + r;
-        ny[r] = row < len ? load_row_pieces(Yg + off + row * 32, yr) : zero;
-        nz[r] = row < len ? load_row_pieces(Zg + off + row * 32, yr) : zero;
+        const bool row_ok = 4 * yr.rowq + r < len;
+        ny[r] = load_row_pieces(reinterpret_cast<const char *>(Yg), xblk + (int64_t)r * xu * 8, y_off, y_ok, row_ok);
+        nz[r] = load_row_pieces(reinterpret_cast<const char *>(Zg), zblk + (int64_t)r * zu * 8, z_off, z_ok, row_ok);
       }
     }
   };
@@ -335,16 +396,19 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       const char *ya = smem + OFF_YN + (32 * qJ + c) * LDN + hh * 16;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
+        if (NARROW && ks * 16 >= fa) continue;  // features past the row width are zeros
         const int T = ks >> 1, u = ks & 1;
-        u32x4 a;
-        a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
-        a.y = E::pack(st[T][8 * u + 2], st[T][8 * u + 3]);
-        a.z = E::pack(st[T][8 * u + 4], st[T][8 * u + 5]);
-        a.w = E::pack(st[T][8 * u + 6], st[T][8 * u + 7]);
         const u32x4 xf0 = lds16(x0 + ks * 32);
         const u32x4 xf1 = lds16(x1 + ks * 32);
-        acc[0] = E::mfma(a, xf0, acc[0]);
-        acc[1] = E::mfma(a, xf1, acc[1]);
+        if (wave_active) {
+          u32x4 a;
+          a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
+          a.y = E::pack(st[T][8 * u + 2], st[T][8 * u + 3]);
+          a.z = E::pack(st[T][8 * u + 4], st[T][8 * u + 5]);
+          a.w = E::pack(st[T][8 * u + 6], st[T][8 * u + 7]);
+          acc[0] = E::mfma(a, xf0, acc[0]);
+          acc[1] = E::mfma(a, xf1, acc[1]);
+        }
         if (q_active) {
           const u32x4 yf = lds16(ya + ks * 32);
           sc = E::mfma(yf, qI ? xf1 : xf0, sc);
@@ -385,29 +449,32 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 
     // (3) intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
     //     (token step outermost, so that consecutive MFMAs write different accumulators)
-    u32x4 zf[4];
+    if (wave_active) {
+      u32x4 zf[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
-    __builtin_amdgcn_s_setprio(1);
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
+      __builtin_amdgcn_s_setprio(1);
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int I = 0; I < 2; ++I) {
-        const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
-        if (needed) {
-          const u32x4 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
-          acc[I] = E::mfma(zf[u], b, acc[I]);
+        for (int I = 0; I < 2; ++I) {
+          const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
+          if (needed) {
+            const u32x4 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
+            acc[I] = E::mfma(zf[u], b, acc[I]);
+          }
         }
-      }
 
-    // (4) state update: St <- l^64 St + (scaled Y)^T Z   (the decay was applied after the sweep)
+      // (4) state update: St <- l^64 St + (scaled Y)^T Z   (the decay was applied after the sweep)
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int T = 0; T < 4; ++T)
-        st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
+        for (int T = 0; T < 4; ++T)
+          if (!NARROW || 32 * T < fa)  // state rows past the width of Y stay zero
+            st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
 
-    __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_s_setprio(0);
+    }
     // (5) stage the output tile (token-major, in the YN region) for coalesced stores
 #pragma unroll
     for (int I = 0; I < 2; ++I)
@@ -420,13 +487,13 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       }
     __syncthreads();  // B: staged output complete; YT / ZT / score no longer read
     {
-      const int64_t off = (int64_t)blk * (BLK * F / 8);
+      const int64_t brow = (int64_t)blk * BLK;
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int row = rowq + 16 * r4;
-        if (!RAGGED || row < len)
+        if (!RAGGED || (row < len && (!NARROW || chunk < ou)))
           __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(smem + OFF_YN + row * LDN + chunk * 16),
-                                      &Og[off + row * 16 + chunk]);
+                                      &Og[(brow + row) * (NARROW ? ou : F / 8) + chunk]);
       }
     }
     if (more) {
@@ -437,20 +504,20 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
   }
 }
 
-template <class E, bool REV, bool TRANS, bool RAGGED>
+template <class E, bool REV, bool TRANS, int MODE>
 __global__ void __launch_bounds__(NTHR, 2)
 la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
          const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
          Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<E, REV, TRANS, RAGGED>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem);
+  apply_body<E, REV, TRANS, MODE>(X, Y, Z, S, states, Out, g, g.d, g.e, (int)blockIdx.x, smem);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
 // work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
 // the triple is spread over block indices 8 apart so that all three land on the same
 // XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
-template <class E, bool RAGGED>
+template <class E, int MODE>
 __global__ void __launch_bounds__(NTHR, 2)
 la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
         const elem16_t *__restrict__ DO, const float *__restrict__ S,
@@ -463,20 +530,22 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    apply_body<E, false, true, RAGGED>(DO, V, K, S, kv_states, DQ, g, item, smem);
+    apply_body<E, false, true, MODE>(DO, V, K, S, kv_states, DQ, g, g.e, g.d, item, smem);
   else if (role == 1)
-    apply_body<E, true, false, RAGGED>(K, Q, DO, S, dkv_states, DV, g, item, smem);
+    apply_body<E, true, false, MODE>(K, Q, DO, S, dkv_states, DV, g, g.d, g.e, item, smem);
   else
-    apply_body<E, true, true, RAGGED>(V, DO, Q, S, dkv_states, DK, g, item, smem);
+    apply_body<E, true, true, MODE>(V, DO, Q, S, dkv_states, DK, g, g.e, g.d, item, smem);
 }
 
 // ------------------------------------------------------------------------------
 // A segment's own state:  causal  sum_b l^(L-b) y_b^T z_b ;  anti-causal  sum_b l^b y_b^T z_b
-// (b from the segment start, L its length), written token-free as 128 x 128 fp32.
-template <class E, bool REV, bool RAGGED>
+// (b from the segment start, L its length), written token-free as 128 x 128 fp32.  Y rows hold
+// g.d features and Z rows g.e (M_NARROW; 128 otherwise).
+template <class E, bool REV, int MODE>
 __global__ void __launch_bounds__(NTHR, 2)
 la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
+  constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -487,9 +556,11 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   const SegWork sw = seg_work(g, (int)blockIdx.x);
   if (sw.seg == skip_seg) return;  // the scan's final segment feeds only the outgoing carry
   const float sl = S[sw.bh % g.h] * LOG2E;
-  const int64_t base = ((int64_t)sw.bh * g.n + sw.tok0) * F;
-  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + base);
-  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + base);
+  const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;
+  const int yw = NARROW ? g.d : F, zw = NARROW ? g.e : F;  // row widths in elements
+  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * yw);
+  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * zw);
+  const int yu = yw / 4, zu = zw / 4;  // 8-byte units per row
 
   const float blockdec = decay(sl, (float)BLK);
   float kdec[4];
@@ -509,15 +580,23 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   // forwards it is the last block, and its tokens sit `len - b` (not 64 - b) before the
   // segment end.
   u32x4 ny[4], nz[4];
+  const uint32_t y_off = lane_offset(yr, 4 * yr.rowq, yu), z_off = lane_offset(yr, 4 * yr.rowq, zu);
+  const PieceMask y_ok = piece_mask(yr, yu), z_ok = piece_mask(yr, zu);
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
-    const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    const u32x4 zero = {0u, 0u, 0u, 0u};
+    const int64_t yblk = (int64_t)blk * BLK * yu * 8, zblk = (int64_t)blk * BLK * zu * 8;  // bytes
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const int row = 4 * yr.rowq + r;
-      ny[r] = (!RAGGED || row < len) ? load_row_pieces(Yg + off + row * 32, yr) : zero;
-      nz[r] = (!RAGGED || row < len) ? load_row_pieces(Zg + off + row * 32, yr) : zero;
+      const bool row_ok = 4 * yr.rowq + r < len;
+      if (!NARROW) {
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        const int64_t row = (int64_t)blk * BLK + 4 * yr.rowq + r;
+        ny[r] = (!RAGGED || row_ok) ? load_row_pieces(Yg + row * 32, yr) : zero;
+        nz[r] = (!RAGGED || row_ok) ? load_row_pieces(Zg + row * 32, yr) : zero;
+      } else {
+        ny[r] = load_row_pieces(reinterpret_cast<const char *>(Yg), yblk + (int64_t)r * yu * 8, y_off, y_ok, row_ok);
+        nz[r] = load_row_pieces(reinterpret_cast<const char *>(Zg), zblk + (int64_t)r * zu * 8, z_off, z_ok, row_ok);
+      }
     }
   };
   auto fill_lds = [&](int buf, int blk) __attribute__((always_inline)) {
@@ -545,16 +624,19 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
     const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
     const char *yt = smem[it & 1];
     const char *zt = yt + F * LDT;
-    u32x4 zf[4];
+    if (!NARROW || 32 * w < g.e) {  // M_NARROW: columns past the width of Z stay zero, as do rows past Y's
+      u32x4 zf[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * w + c, 2 * u + hh));
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * w + c, 2 * u + hh));
 #pragma unroll
-    for (int T = 0; T < 4; ++T) {
+      for (int T = 0; T < 4; ++T) {
+        if (NARROW && 32 * T >= g.d) continue;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
+        for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
-        st[T] = E::mfma(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
+        for (int u = 0; u < 4; ++u)
+          st[T] = E::mfma(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
+      }
     }
     if (more) fill_lds((it + 1) & 1, blk + step);
     __syncthreads();
@@ -585,28 +667,28 @@ int raise_lds(K kernel) {
   return (int)e;
 }
 
-template <class E, bool REV, bool TRANS, bool RAGGED>
+template <class E, bool REV, bool TRANS, int MODE>
 int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
                  void *out, const Geom &g, hipStream_t st) {
-  int rc = raise_lds(la_apply<E, REV, TRANS, RAGGED>);
+  int rc = raise_lds(la_apply<E, REV, TRANS, MODE>);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply<E, REV, TRANS, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
+  la_apply<E, REV, TRANS, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
                                                                  (const elem16_t *)z, s, states,
                                                                  (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
-template <class E, bool RAGGED>
+template <class E, int MODE>
 int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                 hipStream_t st) {
-  int rc = raise_lds(la_bwd3<E, RAGGED>);
+  int rc = raise_lds(la_bwd3<E, MODE>);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3<E, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_bwd3<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                     (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                     kv_states, dkv_states, (elem16_t *)a.dq,
                                                     (elem16_t *)a.dk, (elem16_t *)a.dv, g);
@@ -615,58 +697,77 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
 
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
 // segment it visits last (whose own state feeds nothing else) is skipped.
-template <class E, bool REV, bool RAGGED>
+template <class E, bool REV, int MODE>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, RAGGED><<<grid, NTHR, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
+  la_seg_state<E, REV, MODE><<<grid, NTHR, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
                                                       skip_seg);
   return (int)hipGetLastError();
 }
 
-template <class E, bool RAGGED>
+template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
-    if ((rc = launch_state<E, false, RAGGED>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
-  return launch_apply<E, false, false, RAGGED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
+  return launch_apply<E, false, false, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
 }
 
-template <class E, bool RAGGED>
+template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
   int rc;
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<E, false, RAGGED>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<E, true, RAGGED>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  return launch_bwd3<E, RAGGED>(a, kv_states, dkv_states, g, st);
+  return launch_bwd3<E, MODE>(a, kv_states, dkv_states, g, st);
+}
+
+
+int mode_of(const Geom &g) {
+  if (g.d != F || g.e != F) return M_NARROW;
+  return g.n % BLK != 0 ? M_RAGGED : M_ALIGNED;
+}
+
+template <class E>
+int fwd_m(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  switch (mode_of(g)) {
+    case M_ALIGNED: return fwd_e<E, M_ALIGNED>(a, g, st);
+    case M_RAGGED: return fwd_e<E, M_RAGGED>(a, g, st);
+    default: return fwd_e<E, M_NARROW>(a, g, st);
+  }
+}
+template <class E>
+int bwd_m(const BwdArgs &a, const Geom &g, hipStream_t st) {
+  switch (mode_of(g)) {
+    case M_ALIGNED: return bwd_e<E, M_ALIGNED>(a, g, st);
+    case M_RAGGED: return bwd_e<E, M_RAGGED>(a, g, st);
+    default: return bwd_e<E, M_NARROW>(a, g, st);
+  }
 }
 
 }  // namespace
 
 int mfma_fwd(const FwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
-  const bool ragged = g.n % BLK != 0;
-  if (dtype == LASP_DTYPE_F16) return ragged ? fwd_e<ElemF16, true>(a, g, st) : fwd_e<ElemF16, false>(a, g, st);
-  return ragged ? fwd_e<ElemBF16, true>(a, g, st) : fwd_e<ElemBF16, false>(a, g, st);
+  return dtype == LASP_DTYPE_F16 ? fwd_m<ElemF16>(a, g, st) : fwd_m<ElemBF16>(a, g, st);
 }
 
 int mfma_bwd(const BwdArgs &a, const Geom &g, int dtype, hipStream_t st) {
-  const bool ragged = g.n % BLK != 0;
-  if (dtype == LASP_DTYPE_F16) return ragged ? bwd_e<ElemF16, true>(a, g, st) : bwd_e<ElemF16, false>(a, g, st);
-  return ragged ? bwd_e<ElemBF16, true>(a, g, st) : bwd_e<ElemBF16, false>(a, g, st);
+  return dtype == LASP_DTYPE_F16 ? bwd_m<ElemF16>(a, g, st) : bwd_m<ElemBF16>(a, g, st);
 }
 
 }  // namespace lasp

@@ -80,7 +80,11 @@ def test_kernel_path_selection(lib):
     assert _abi.kernel_path(1, 16, 65520, 128, 128, torch.float32) == _abi.PATH_MFMA   # ragged: masked tail
     assert _abi.kernel_path(1, 16, 65536, 128, 64, torch.float32) == _abi.PATH_GENERIC
     assert _abi.kernel_path(1, 16, 65500, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
-    assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_MFMA    # rows read zero-extended
+    assert _abi.kernel_path(1, 16, 65536, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC  # not a multiple of 8
+    # a state is stored zero-extended to 128 x 128 on the MFMA path, d x e on the generic one
+    assert _abi.plan(1, 2, 256, 64, 128, torch.bfloat16, 256)[2] == 2 * 128 * 128 * 4
+    assert _abi.plan(1, 2, 256, 64, 128, torch.float32, 256)[2] == 2 * 64 * 128 * 4
 
 
 def test_null_and_workspace_errors_need_no_gpu(lib):

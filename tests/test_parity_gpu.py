@@ -41,7 +41,8 @@ def test_library_loaded_and_path_selection(gpu_device):
     assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 96, torch.float32) == _abi.PATH_GENERIC
     assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
-    assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_GENERIC
+    assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(2, 12, 2048, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC
 
 
 @pytest.mark.parametrize("state", [False, True])
@@ -59,8 +60,8 @@ def test_generic_fp32_small(gpu_device, shape, state):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_generic_low_precision_io(gpu_device, dtype):
-    # e != d handed to the library as is: generic kernels with 16-bit I/O
-    inp = make_inputs(2, 12, 500, 128, 64, dtype, seed=3, state=True, state_std=1.0)
+    # e not a multiple of 8, handed to the library as is: generic kernels with 16-bit I/O
+    inp = make_inputs(2, 12, 500, 128, 60, dtype, seed=3, state=True, state_std=1.0)
     s = O.slopes_alibi(12)
     got = run_abi(inp, s, gpu_device, exact=True)
     check(got, oracle(inp, s), TOL[dtype], what=str(dtype))
@@ -158,15 +159,46 @@ def test_mfma_cached_states_equal_recompute(gpu_device):
         assert torch.equal(a[name], c[name]), name
 
 
-@pytest.mark.parametrize("d,e", [(128, 64), (64, 128), (64, 64), (96, 32)])
-def test_narrow_bf16_heads_run_padded_on_mfma(gpu_device, d, e):
-    # the reference's own test shape has e = 64 (tests/test.py:95): zero-padded to 128, exact
+@pytest.mark.parametrize("d,e", [(128, 64), (64, 128), (64, 64), (96, 32), (8, 120), (100, 36)])
+def test_narrow_bf16_heads_on_mfma(gpu_device, d, e):
+    """Narrow heads: the kernels read rows zero-extended when d and e are multiples of 8 (the reference's
+    own test shape has e = 64, tests/test.py:95); otherwise the Python layer zero-pads.  Exact either way."""
+    from lasp_amd import _abi
+
+    native = d % 8 == 0 and e % 8 == 0
+    assert _abi.kernel_path(2, 3, 512, d, e, torch.bfloat16) == (_abi.PATH_MFMA if native else _abi.PATH_GENERIC)
     inp = make_inputs(2, 3, 512, d, e, torch.bfloat16, seed=d + e, state=True, state_std=1.0)
+    assert _abi._pad_to_mfma(inp["q"], inp["v"]) == (not native)
     s = O.slopes_alibi(3)
     for cache in (False, True):
         got = run_abi(inp, s, gpu_device, seg_len=128, cache=cache)
         assert got["o"].shape[-1] == e and got["dq"].shape[-1] == d and got["kv_out"].shape[-2:] == (d, e)
-        check(got, oracle(inp, s), 2e-2, what=f"padded d={d} e={e} cache={cache}")
+        check(got, oracle(inp, s), 2e-2, what=f"narrow d={d} e={e} cache={cache}")
+
+
+def test_narrow_rows_leave_neighbouring_memory_alone(gpu_device):
+    """Outputs narrower than 128 features are written at their own width: a guard band after
+    each output tensor keeps its bits."""
+    from lasp_amd import _abi
+
+    b, h, n, d, e = 1, 2, 200, 64, 32
+    inp = make_inputs(b, h, n, d, e, torch.bfloat16, seed=77, state=True, state_std=1.0, device=gpu_device)
+    s = O.slopes_alibi(h).to(gpu_device)
+    o, states, sl = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=torch.empty_like(inp["kv"]))
+    torch.cuda.synchronize()
+    # re-run into views of guarded buffers through the raw entry point
+    lib = _abi.load()
+    guard = 4096
+    buf = torch.full((b * h * n * e + guard,), 1.5, dtype=torch.bfloat16, device=gpu_device)
+    kvo = torch.full((b * h * d * e + guard,), -2.5, dtype=torch.float32, device=gpu_device)
+    rc = lib.lasp_chunk_fwd(inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(),
+                            inp["kv"].data_ptr(), kvo.data_ptr(), buf.data_ptr(), states.data_ptr(),
+                            b, h, n, d, e, _abi.DTYPE_CODE[torch.bfloat16], sl,
+                            torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0
+    assert torch.equal(buf[:b * h * n * e].view(b, h, n, e), o)
+    assert (buf[b * h * n * e:] == 1.5).all() and (kvo[b * h * d * e:] == -2.5).all()
 
 
 @pytest.mark.parametrize("n,d,e", [(2047, 128, 128), (65, 128, 128), (700, 128, 64), (63, 128, 128), (1, 128, 128)])
