@@ -235,9 +235,9 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 // ------------------------------------------------------------------------------
 // M_RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
 // partial.  M_NARROW: in addition X and Y rows hold `fa` features, Z and Out rows `fb`
-// (multiples of 8, at most 128); feature steps, state tiles and waves that would only see the
-// zero extension are skipped.  M_ALIGNED carries none of that bookkeeping; fa and fb are read
-// in M_NARROW only.
+// (multiples of 8, at most 128); the upper half of the feature steps and state tiles, and waves
+// whose columns lie in the zero extension, are skipped when they would only see zeros.
+// M_ALIGNED carries none of that bookkeeping; fa and fb are read in M_NARROW only.
 template <class E, bool REV, bool TRANS, int MODE>
 __device__ __forceinline__ void
 apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
@@ -394,9 +394,11 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       const char *x0 = smem + OFF_XN + c * LDN + hh * 16;
       const char *x1 = x0 + 32 * LDN;
       const char *ya = smem + OFF_YN + (32 * qJ + c) * LDN + hh * 16;
+      // M_NARROW: the upper 64 features are skipped as a whole when the rows are no wider
+      const bool upper_half = !NARROW || fa > 64;
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        if (NARROW && ks * 16 >= fa) continue;  // features past the row width are zeros
+        if (ks >= 4 && !upper_half) continue;
         const int T = ks >> 1, u = ks & 1;
         const u32x4 xf0 = lds16(x0 + ks * 32);
         const u32x4 xf1 = lds16(x1 + ks * 32);
@@ -470,7 +472,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       for (int u = 0; u < 4; ++u)
 #pragma unroll
         for (int T = 0; T < 4; ++T)
-          if (!NARROW || 32 * T < fa)  // state rows past the width of Y stay zero
+          if (!NARROW || T < 2 || fa > 64)  // state rows past the width of Y stay zero
             st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
 
       __builtin_amdgcn_s_setprio(0);
@@ -630,7 +632,7 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
       for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * w + c, 2 * u + hh));
 #pragma unroll
       for (int T = 0; T < 4; ++T) {
-        if (NARROW && 32 * T >= g.d) continue;
+        if (NARROW && T >= 2 && g.d <= 64) continue;
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
