@@ -10,6 +10,7 @@ stream, like the Triton launches it replaces
 from __future__ import annotations
 
 import ctypes
+import functools
 import os
 from typing import Optional, Tuple
 
@@ -100,8 +101,9 @@ def _check_state(name, t, b, h, d, e):
                         f"got {t.dtype} {tuple(t.shape)}")
 
 
+@functools.lru_cache(maxsize=256)
 def plan(b: int, h: int, n: int, d: int, e: int, dtype: torch.dtype, seg_len: int = 0) -> Tuple[int, int, int]:
-    """(seg_len, n_seg, bytes of one segment-state array) for a shape."""
+    """(seg_len, n_seg, bytes of one segment-state array) for a shape (a pure function of its arguments)."""
     lib = load()
     sl, ns, sb = _c_int(0), _c_int(0), _c_size(0)
     rc = lib.lasp_plan(b, h, n, d, e, DTYPE_CODE[dtype], seg_len, ctypes.byref(sl), ctypes.byref(ns), ctypes.byref(sb))

@@ -45,3 +45,7 @@ if __name__ == "__main__":
     make("generic_f32_b1_h2_n150_d32_e16", 1, 2, 150, 32, 16, torch.float32, 101, [0.25, 0.02])
     # bf16 I/O on the MFMA shape, two blocks
     make("mfma_bf16_b1_h1_n128_d128_e128", 1, 1, 128, 128, 128, torch.bfloat16, 102, [0.0625])
+    # bf16 I/O with narrow value rows (the reference's own test has e = 64) and a ragged length
+    make("mfma_bf16_b1_h2_n100_d128_e64", 1, 2, 100, 128, 64, torch.bfloat16, 103, [0.5, 0.0039])
+    # fp32 I/O on the fp32 MFMA shape, ragged length
+    make("mfma_f32_b1_h1_n80_d128_e128", 1, 1, 80, 128, 128, torch.float32, 104, [0.125])
