@@ -13,6 +13,20 @@
  *     kv_in, kv_out, dkv_in, dkv_out : (b, h, d, e) float, may be NULL
  *     seg states   : (b, h, n_seg, d, e) float workspace (see lasp_plan)
  *
+ * Alignment: q, k, v, o, do, dq, dk, dv start on a 16-byte boundary (the kernels
+ * fetch rows with 8-byte loads and store them with 16-byte stores; rows of d or e
+ * 16-bit elements with d, e multiples of 8 keep every row aligned as well); s, the
+ * states and the workspaces on a 4-byte boundary.  A pointer that is not returns
+ * LASP_E_ALIGN.
+ * Device: the calling thread's current device (hipSetDevice) must be the one that
+ * owns every pointer and `stream`; the calls check this for q (LASP_E_DEVICE) and
+ * never switch devices themselves.
+ * Range: the 16-bit kernels round the fp32 states, the decayed keys and the masked
+ * q.k scores to the I/O element type before each matrix product (accumulation is
+ * fp32).  With fp16 I/O any of them beyond 65504 in magnitude becomes inf -- a large
+ * caller-supplied kv_in, or a slow-decay head with positive-mean feature maps over a
+ * long chunk; bf16 has the range of fp32 and no such limit.
+ *
  * Every call only ENQUEUES work on `stream` (a hipStream_t; NULL = the default
  * stream); nothing is allocated, freed or synchronised, pointers are borrowed
  * until the enqueued work has run.  Return value: 0 on success, > 0 a
@@ -52,6 +66,8 @@ extern "C" {
 #define LASP_E_DTYPE (-3)    /* unknown dtype code */
 #define LASP_E_SEGMENT (-4)  /* seg_len invalid for this shape */
 #define LASP_E_WORKSPACE (-5)/* workspace missing or too small */
+#define LASP_E_ALIGN (-6)    /* a pointer is not aligned as the tensor contract asks */
+#define LASP_E_DEVICE (-7)   /* q is not device memory of the calling thread's current device */
 
 /* Which kernel family a shape/dtype is served by (lasp_kernel_path). */
 #define LASP_PATH_GENERIC 0 /* fp32-FMA kernels: any dtype, any n, d,e <= 128 */
@@ -122,7 +138,9 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
  * max_launches of them; later launches go untimed).  lasp_profile_end waits for
  * the recorded events and returns, per kernel class, the summed duration in
  * milliseconds and the number of launches (arrays of LASP_KERNEL_CLASSES
- * entries; either may be NULL).  One profile at a time, one thread.
+ * entries; either may be NULL).  One profile at a time; launches may come from
+ * any thread while it is open (each claims its slot atomically), begin and end
+ * are called by one thread.
  */
 #define LASP_KERNEL_CLASSES 5
 #define LASP_KC_APPLY 0   /* la_apply: the block sweep producing O */

@@ -151,7 +151,28 @@ def _shapes(q, k, v):
 def _slopes(s: torch.Tensor, h: int, dev) -> torch.Tensor:
     if s.numel() != h:
         raise LaspError(f"need {h} slopes, got a tensor with {s.numel()} elements")
+    if s.dtype == torch.float32 and s.device == dev and s.is_contiguous():
+        return s  # the usual case costs nothing; data_ptr() does not care about autograd
     return s.detach().to(device=dev, dtype=torch.float32).contiguous()
+
+
+class _on_device:
+    """`with torch.cuda.device(dev)` only when dev is not already current (backward runs on autograd's
+    thread, which PyTorch has already switched to the right device)."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, dev):
+        self.guard = None if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
@@ -169,7 +190,7 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     _check_state("kv_in", kv_in, b, h, d, e)
     _check_state("kv_out", kv_out, b, h, d, e)
     seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
         states = None
         if n_seg > 1 or kv_in is not None or kv_out is not None:
@@ -202,15 +223,18 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
             raise LaspError(f"kv_seg_states must be the contiguous float32 array of {state_bytes} bytes that "
                             f"chunk_fwd returned for this shape, got {kv_seg_states.dtype} "
                             f"{tuple(kv_seg_states.shape)}")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
-        n_arrays = 2 if kv_seg_states is None else 1
-        ws = torch.empty((n_arrays * state_bytes // 4,), dtype=torch.float32, device=dev)
+        # one state array for the dKV scan, one more when the KV states have to be rebuilt
+        need_dkv = n_seg > 1 or dkv_in is not None or dkv_out is not None
+        need_kv = kv_seg_states is None and (n_seg > 1 or kv_in is not None)
+        n_arrays = int(need_dkv) + int(need_kv)
+        ws = torch.empty((n_arrays * state_bytes // 4,), dtype=torch.float32, device=dev) if n_arrays else None
         rc = lib.lasp_chunk_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), _ptr(kv_in),
                                 _ptr(dkv_in), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _ptr(dkv_out),
-                                _ptr(kv_seg_states), ws.data_ptr(), ws.numel() * 4, b, h, n, d, e,
+                                _ptr(kv_seg_states), _ptr(ws), n_arrays * state_bytes, b, h, n, d, e,
                                 DTYPE_CODE[q.dtype], seg_len, torch.cuda.current_stream(dev).cuda_stream)
     if rc:
         _raise(rc, "lasp_chunk_bwd")

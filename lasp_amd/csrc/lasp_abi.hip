@@ -3,6 +3,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "lasp_common.h"
 
 namespace lasp {
@@ -21,17 +23,32 @@ struct ProfEntry {
   int cls;
   hipEvent_t start, stop;
 };
-static ProfEntry *g_prof = nullptr;  // non-NULL while a profile is open
-static int g_prof_cap = 0, g_prof_used = 0;
+// Launches may come from several threads (PyTorch runs backward on its own thread): a launch
+// claims its slot with one atomic increment, and lasp_profile_end only reads slots after the
+// profile has been closed to new launches and the claimed ones have recorded their events.
+static std::atomic<ProfEntry *> g_prof{nullptr};  // non-NULL while a profile is open
+static std::atomic<int> g_prof_used{0};           // slots claimed (may run past the capacity)
+static std::atomic<int> g_prof_busy{0};           // launches between claiming a slot and recording its stop event
+static int g_prof_cap = 0;
 
-ProfScope::ProfScope(int kernel_class, hipStream_t st) : slot(-1), stream(st) {
-  if (!g_prof || g_prof_used >= g_prof_cap) return;
-  slot = g_prof_used++;
-  g_prof[slot].cls = kernel_class;
-  (void)hipEventRecord(g_prof[slot].start, stream);
+ProfScope::ProfScope(int kernel_class, hipStream_t st) : slot(-1), entry(nullptr), stream(st) {
+  if (!g_prof.load(std::memory_order_acquire)) return;
+  g_prof_busy.fetch_add(1, std::memory_order_acq_rel);
+  ProfEntry *p = g_prof.load(std::memory_order_acquire);  // re-read: the profile may have closed meanwhile
+  const int claimed = p ? g_prof_used.fetch_add(1, std::memory_order_acq_rel) : -1;
+  if (!p || claimed >= g_prof_cap) {
+    g_prof_busy.fetch_sub(1, std::memory_order_acq_rel);
+    return;
+  }
+  slot = claimed;
+  entry = p + slot;
+  entry->cls = kernel_class;
+  (void)hipEventRecord(entry->start, stream);
 }
 ProfScope::~ProfScope() {
-  if (slot >= 0) (void)hipEventRecord(g_prof[slot].stop, stream);
+  if (slot < 0) return;
+  (void)hipEventRecord(entry->stop, stream);
+  g_prof_busy.fetch_sub(1, std::memory_order_acq_rel);
 }
 
 namespace {
@@ -114,6 +131,36 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   return 0;
 }
 
+// The kernels fetch rows of q/k/v/do with 8-byte loads and store o/dq/dk/dv with 16-byte stores,
+// and read states as floats: tensors must start on a 16-byte boundary, states on a 4-byte one.
+int check_aligned(const char *call, const char *name, const void *p, size_t align) {
+  if (p && ((uintptr_t)p % align) != 0) {
+    set_error("%s: %s = %p is not aligned to %zu bytes", call, name, p, align);
+    return LASP_E_ALIGN;
+  }
+  return 0;
+}
+
+// The calling thread's current device must be the one that owns the tensors (checked on q).
+int check_device(const char *call, const void *q) {
+  hipPointerAttribute_t attr;
+  hipError_t e = hipPointerGetAttributes(&attr, q);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // the failed query must not be reported by a later launch
+    set_error("%s: q = %p is not a device pointer known to HIP (%s)", call, q, hipGetErrorString(e));
+    return LASP_E_DEVICE;
+  }
+  int dev = -1;
+  e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (attr.type != hipMemoryTypeDevice || attr.device != dev) {
+    set_error("%s: q = %p lives on device %d (memory type %d) but the calling thread's current device is %d",
+              call, q, attr.device, (int)attr.type, dev);
+    return LASP_E_DEVICE;
+  }
+  return 0;
+}
+
 size_t state_bytes_of(const Geom &g) {
   return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.sd * g.se;
 }
@@ -130,7 +177,7 @@ int lasp_abi_version(void) { return LASP_ABI_VERSION; }
 const char *lasp_last_error(void) { return g_err; }
 
 int lasp_profile_begin(int max_launches) {
-  if (g_prof) {
+  if (g_prof.load()) {
     set_error("lasp_profile_begin: a profile is already open");
     return LASP_E_SHAPE;
   }
@@ -154,24 +201,26 @@ int lasp_profile_begin(int max_launches) {
     }
   }
   g_prof_cap = max_launches;
-  g_prof_used = 0;
-  g_prof = p;
+  g_prof_used.store(0);
+  g_prof.store(p, std::memory_order_release);
   return 0;
 }
 
 int lasp_profile_end(double *ms_per_class, int *launches_per_class) {
-  if (!g_prof) {
+  ProfEntry *p = g_prof.exchange(nullptr, std::memory_order_acq_rel);
+  if (!p) {
     set_error("lasp_profile_end: no profile is open");
     return LASP_E_SHAPE;
   }
-  ProfEntry *p = g_prof;
-  g_prof = nullptr;
+  while (g_prof_busy.load(std::memory_order_acquire) > 0) {
+  }  // a launch on another thread is between its two event records
+  const int used = g_prof_used.load() < g_prof_cap ? g_prof_used.load() : g_prof_cap;
   for (int c = 0; c < KC_COUNT; ++c) {
     if (ms_per_class) ms_per_class[c] = 0.0;
     if (launches_per_class) launches_per_class[c] = 0;
   }
   int rc = 0;
-  for (int i = 0; i < g_prof_used; ++i) {
+  for (int i = 0; i < used; ++i) {
     float ms = 0.f;
     hipError_t e = hipEventSynchronize(p[i].stop);
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, p[i].start, p[i].stop);
@@ -184,7 +233,8 @@ int lasp_profile_end(double *ms_per_class, int *launches_per_class) {
     (void)hipEventDestroy(p[i].stop);
   }
   delete[] p;
-  g_prof_cap = g_prof_used = 0;
+  g_prof_cap = 0;
+  g_prof_used.store(0);
   if (rc) set_error("lasp_profile_end: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
   return rc;
 }
@@ -207,6 +257,26 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
   return (mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
 }
 
+static int chunk_fwd_impl(const char *me, const void *q, const void *k, const void *v, const float *s,
+                          const float *kv_in, float *kv_out, void *o, float *seg_states, const Geom &g,
+                          int dtype, void *stream) {
+  int rc;
+  if ((rc = check_aligned(me, "q", q, 16)) || (rc = check_aligned(me, "k", k, 16)) ||
+      (rc = check_aligned(me, "v", v, 16)) || (rc = check_aligned(me, "o", o, 16)) ||
+      (rc = check_aligned(me, "s", s, 4)) || (rc = check_aligned(me, "kv_in", kv_in, 4)) ||
+      (rc = check_aligned(me, "kv_out", kv_out, 4)) || (rc = check_aligned(me, "seg_states", seg_states, 4)))
+    return rc;
+  if ((rc = check_device(me, q))) return rc;
+  (void)hipGetLastError();  // an earlier, unrelated error of this thread is not this call's
+  FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
+  hipStream_t st = (hipStream_t)stream;
+  rc = mfma_eligible(g.d, g.e, dtype)       ? mfma_fwd(a, g, dtype, st)
+       : mfma_f32_eligible(g.d, g.e, dtype) ? mfma_f32_fwd(a, g, st)
+                                            : generic_fwd(a, g, dtype, st);
+  if (rc > 0) set_error("%s: HIP error %d: %s", me, rc, hipGetErrorString((hipError_t)rc));
+  return rc;
+}
+
 int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, const float *kv_in,
                    float *kv_out, void *o, float *seg_states, int b, int h, int64_t n, int d, int e,
                    int dtype, int seg_len, void *stream) {
@@ -222,13 +292,7 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
               state_bytes_of(g), g.n_seg, (kv_in || kv_out) ? " with KV in/out" : "");
     return LASP_E_WORKSPACE;
   }
-  FwdArgs a{q, k, v, s, kv_in, kv_out, o, seg_states};
-  hipStream_t st = (hipStream_t)stream;
-  rc = mfma_eligible(d, e, dtype)       ? mfma_fwd(a, g, dtype, st)
-       : mfma_f32_eligible(d, e, dtype) ? mfma_f32_fwd(a, g, st)
-                                        : generic_fwd(a, g, dtype, st);
-  if (rc > 0) set_error("lasp_chunk_fwd: HIP error %d: %s", rc, hipGetErrorString((hipError_t)rc));
-  return rc;
+  return chunk_fwd_impl("lasp_chunk_fwd", q, k, v, s, kv_in, kv_out, o, seg_states, g, dtype, stream);
 }
 
 int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, const void *d_o,
@@ -252,6 +316,18 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
               workspace ? workspace_bytes : (size_t)0);
     return LASP_E_WORKSPACE;
   }
+  const char *me = "lasp_chunk_bwd";
+  if ((rc = check_aligned(me, "q", q, 16)) || (rc = check_aligned(me, "k", k, 16)) ||
+      (rc = check_aligned(me, "v", v, 16)) || (rc = check_aligned(me, "do", d_o, 16)) ||
+      (rc = check_aligned(me, "dq", dq, 16)) || (rc = check_aligned(me, "dk", dk, 16)) ||
+      (rc = check_aligned(me, "dv", dv, 16)) || (rc = check_aligned(me, "s", s, 4)) ||
+      (rc = check_aligned(me, "kv_in", kv_in, 4)) || (rc = check_aligned(me, "dkv_in", dkv_in, 4)) ||
+      (rc = check_aligned(me, "dkv_out", dkv_out, 4)) ||
+      (rc = check_aligned(me, "kv_seg_states", kv_seg_states, 4)) ||
+      (rc = check_aligned(me, "workspace", workspace, 4)))
+    return rc;
+  if ((rc = check_device(me, q))) return rc;
+  (void)hipGetLastError();  // an earlier, unrelated error of this thread is not this call's
   BwdArgs a{q,  k,  v,       s,
             d_o, kv_in, dkv_in, dq,
             dk, dv, dkv_out, kv_seg_states,

@@ -97,13 +97,30 @@ int launch_segment_scan(float *states, const float *carry_in, float *carry_out,
 
 void set_error(const char *fmt, ...);
 
+// Dynamic LDS above the default limit has to be granted once per kernel and device.  The grant is
+// always for the kernel's maximum (so callers with different shapes cannot lower each other's
+// limit between the grant and the launch) and is remembered per kernel, thread and device.
+template <auto Kernel>
+int grant_lds(int max_bytes) {
+  static thread_local uint64_t granted = 0;  // one bit per device ordinal below 64
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev >= 0 && dev < 64 && ((granted >> dev) & 1u)) return 0;
+  e = hipFuncSetAttribute((const void *)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, max_bytes);
+  if (e == hipSuccess && dev >= 0 && dev < 64) granted |= (uint64_t)1 << dev;
+  return (int)e;
+}
+
 // Optional per-kernel timing (lasp_profile_begin / lasp_profile_end): while a
 // profile is open every kernel launch is bracketed by two events on its stream.
 enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_BWD3 = 4, KC_COUNT = 5 };
+struct ProfEntry;
 struct ProfScope {
   ProfScope(int kernel_class, hipStream_t st);
   ~ProfScope();
   int slot;
+  ProfEntry *entry;
   hipStream_t stream;
 };
 

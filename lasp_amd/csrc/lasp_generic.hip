@@ -361,11 +361,8 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   if (carry_out && in_carry) carry_out[cidx] = run;
 }
 
-template <class K>
-int set_lds(K kernel, size_t bytes) {
-  return (int)hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)bytes);
-}
+// the largest dynamic LDS any kernel of this family asks for (generic_bwd_dkdv at d = e = 128)
+constexpr int GENERIC_MAX_LDS = (int)sizeof(float) * (4 * GB * 129 + 2 * GB * LDS_S + 128 * 129 + 2 * GB);
 
 template <class T>
 int fwd_t(const FwdArgs &a, const Geom &g, hipStream_t st) {
@@ -375,7 +372,7 @@ int fwd_t(const FwdArgs &a, const Geom &g, hipStream_t st) {
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
     const size_t lds = sizeof(float) * (GB * ldd + GB * lde + d * lde + 2 * GB);
-    if ((rc = set_lds(generic_seg_state<T>, lds))) return rc;
+    if ((rc = grant_lds<generic_seg_state<T>>(GENERIC_MAX_LDS))) return rc;
     {
       ProfScope prof(KC_GENERIC, st);
       generic_seg_state<T><<<grid, NT, lds, st>>>((const T *)a.k, (const T *)a.v, a.s, a.seg_states, g, 0);
@@ -383,7 +380,7 @@ int fwd_t(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
   const size_t lds = sizeof(float) * (2 * GB * ldd + GB * lde + GB * LDS_S + d * lde + 2 * GB);
-  if ((rc = set_lds(generic_fwd_apply<T>, lds))) return rc;
+  if ((rc = grant_lds<generic_fwd_apply<T>>(GENERIC_MAX_LDS))) return rc;
   ProfScope prof(KC_GENERIC, st);
   generic_fwd_apply<T><<<grid, NT, lds, st>>>((const T *)a.q, (const T *)a.k, (const T *)a.v, a.s,
                                               need_states ? a.seg_states : nullptr, (T *)a.o, g);
@@ -396,7 +393,7 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   int rc;
   const size_t lds_state = sizeof(float) * (GB * ldd + GB * lde + d * lde + 2 * GB);
-  if ((rc = set_lds(generic_seg_state<T>, lds_state))) return rc;
+  if ((rc = grant_lds<generic_seg_state<T>>(GENERIC_MAX_LDS))) return rc;
 
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
@@ -418,7 +415,7 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
   }
   {
     const size_t lds = sizeof(float) * (2 * GB * lde + GB * ldd + GB * LDS_S + d * lde + 2 * GB);
-    if ((rc = set_lds(generic_bwd_dq<T>, lds))) return rc;
+    if ((rc = grant_lds<generic_bwd_dq<T>>(GENERIC_MAX_LDS))) return rc;
     ProfScope prof(KC_GENERIC, st);
     generic_bwd_dq<T><<<grid, NT, lds, st>>>((const T *)a.k, (const T *)a.v, (const T *)a.d_o, a.s,
                                              kv_states, (T *)a.dq, g);
@@ -426,7 +423,7 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
   {
     const size_t lds =
         sizeof(float) * (2 * GB * ldd + 2 * GB * lde + 2 * GB * LDS_S + d * lde + 2 * GB);
-    if ((rc = set_lds(generic_bwd_dkdv<T>, lds))) return rc;
+    if ((rc = grant_lds<generic_bwd_dkdv<T>>(GENERIC_MAX_LDS))) return rc;
     ProfScope prof(KC_GENERIC, st);
     generic_bwd_dkdv<T><<<grid, NT, lds, st>>>((const T *)a.q, (const T *)a.k, (const T *)a.v,
                                                (const T *)a.d_o, a.s, dkv_states, (T *)a.dk,

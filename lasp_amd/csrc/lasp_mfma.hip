@@ -652,27 +652,10 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
       sp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
 }
 
-// Dynamic LDS above the default limit has to be granted once per kernel and device.
-template <class K>
-int raise_lds(K kernel) {
-  static thread_local const void *granted_fn = nullptr;
-  static thread_local int granted_dev = -1;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return (int)e;
-  if (granted_fn == (const void *)kernel && granted_dev == dev) return 0;
-  e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, APPLY_LDS);
-  if (e == hipSuccess) {
-    granted_fn = (const void *)kernel;
-    granted_dev = dev;
-  }
-  return (int)e;
-}
-
 template <class E, bool REV, bool TRANS, int MODE>
 int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
                  void *out, const Geom &g, hipStream_t st) {
-  int rc = raise_lds(la_apply<E, REV, TRANS, MODE>);
+  int rc = grant_lds<la_apply<E, REV, TRANS, MODE>>(APPLY_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
@@ -685,7 +668,7 @@ int launch_apply(const void *x, const void *y, const void *z, const float *s, co
 template <class E, int MODE>
 int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                 hipStream_t st) {
-  int rc = raise_lds(la_bwd3<E, MODE>);
+  int rc = grant_lds<la_bwd3<E, MODE>>(APPLY_LDS);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);

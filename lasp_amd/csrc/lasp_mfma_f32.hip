@@ -378,22 +378,6 @@ la32_seg_state(const float *__restrict__ Y, const float *__restrict__ Z, const f
       sp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
 }
 
-template <class K>
-int raise_lds(K kernel) {
-  static thread_local const void *granted_fn = nullptr;
-  static thread_local int granted_dev = -1;
-  int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return (int)e;
-  if (granted_fn == (const void *)kernel && granted_dev == dev) return 0;
-  e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, APPLY_LDS);
-  if (e == hipSuccess) {
-    granted_fn = (const void *)kernel;
-    granted_dev = dev;
-  }
-  return (int)e;
-}
-
 template <bool REV, bool RAGGED>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
@@ -413,7 +397,7 @@ int fwd_r(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_state<false, RAGGED>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
-  if ((rc = raise_lds(la32_apply<false, false, RAGGED>))) return rc;
+  if ((rc = grant_lds<la32_apply<false, false, RAGGED>>(APPLY_LDS))) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
   la32_apply<false, false, RAGGED><<<grid, NTHR, APPLY_LDS, st>>>((const float *)a.q, (const float *)a.k,
@@ -438,7 +422,7 @@ int bwd_r(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  if ((rc = raise_lds(la32_bwd3<RAGGED>))) return rc;
+  if ((rc = grant_lds<la32_bwd3<RAGGED>>(APPLY_LDS))) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);

@@ -38,7 +38,7 @@ class LaspFuseParallel(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, s, KV, DKV):
-        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, True, True)
+        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, True, True, True)
 
     @staticmethod
     def backward(ctx, do):
@@ -51,4 +51,4 @@ lasp_fuse_parallel_ = LaspFuseParallel.apply
 def lasp_fuse_parallel(q, k, v, ed, KV, DKV):
     if q.shape[-1] <= 128:
         return lasp_fuse_parallel_(q, k, v, ed, KV, DKV)
-    return run_sliced(q, k, v, ed, KV, DKV, True, True)
+    return run_sliced(q, k, v, ed, KV, DKV, True, True, True)

@@ -20,6 +20,7 @@ Two modes:
 from __future__ import annotations
 
 import operator
+from collections import deque
 from functools import reduce
 from typing import Dict, Optional, Tuple
 
@@ -35,7 +36,7 @@ __all__ = [
     "get_data_parallel_world_size", "get_data_parallel_rank",
     "get_seq_parallel_send_rank", "get_seq_parallel_receive_rank",
     "get_global_memory_buffer", "destroy_global_memory_buffer", "destroy_parallel_groups",
-    "get_rank", "GlobalMemoryBuffer", "LoopbackGroup", "state_send", "state_recv", "loopback_pending",
+    "get_rank", "GlobalMemoryBuffer", "LoopbackGroup", "state_send", "state_recv", "state_take", "loopback_pending",
 ]
 
 
@@ -44,7 +45,8 @@ class LoopbackGroup:
 
     def __init__(self, size: int):
         self.size = int(size)
-        self.mailbox: Dict[Tuple[int, int], torch.Tensor] = {}
+        # (src, dst, tag) -> states in the order they were sent; an emptied queue is removed
+        self.mailbox: Dict[Tuple[int, int, int], deque] = {}
 
     def __repr__(self):
         return f"LoopbackGroup(size={self.size}, pending={sorted(self.mailbox)})"
@@ -208,34 +210,69 @@ def get_rank(group):
 
 
 # ---------------------------------------------------------------- state passing
-def state_send(tensor: torch.Tensor, dst: int, group, src: Optional[int] = None) -> None:
-    """Hands a d x e state to rank `dst` (dist.send, or the loopback mailbox)."""
+# The loopback mailbox is first-in first-out per (sender, receiver, tag), as dist.send / dist.recv
+# are per pair of ranks: an operator on wide heads sends one state per feature slice to the same
+# neighbour before that neighbour receives any of them.  `tag` (the feature-slice index) only
+# exists in the loopback; over torch.distributed the order of the calls pairs the messages.
+def state_send(tensor: torch.Tensor, dst: int, group, src: Optional[int] = None, tag: int = 0,
+               give: bool = False) -> None:
+    """Hands a d x e state to rank `dst` (dist.send, or the loopback mailbox).
+
+    The mailbox keeps a copy, unless the sender gives the tensor away (`give`: it will not touch
+    it again)."""
     if isinstance(group, LoopbackGroup):
         me = get_sequence_parallel_rank() if src is None else src
-        group.mailbox[(me, dst)] = tensor.detach().clone()
+        t = tensor.detach()
+        group.mailbox.setdefault((me, dst, tag), deque()).append(t if give else t.clone())
         return
     dist.send(tensor, dst=dst, group=group)
 
 
-def state_recv(tensor: torch.Tensor, src: int, group, dst: Optional[int] = None) -> None:
+def _loopback_pop(group: LoopbackGroup, src: int, me: int, tag: int) -> torch.Tensor:
+    key = (src, me, tag)
+    queue = group.mailbox.get(key)
+    if not queue:
+        raise RuntimeError(
+            f"loopback recv on rank {me}: nothing was sent by rank {src} "
+            f"(pending: {loopback_pending()}); chunks must run in chain order"
+        )
+    t = queue.popleft()
+    if not queue:
+        del group.mailbox[key]
+    return t
+
+
+def state_recv(tensor: torch.Tensor, src: int, group, dst: Optional[int] = None, tag: int = 0) -> None:
     """Fills `tensor` with the state rank `src` sent (dist.recv, or the mailbox)."""
     if isinstance(group, LoopbackGroup):
         me = get_sequence_parallel_rank() if dst is None else dst
-        key = (src, me)
-        if key not in group.mailbox:
-            raise RuntimeError(
-                f"loopback recv on rank {me}: nothing was sent by rank {src} "
-                f"(pending: {sorted(group.mailbox)}); chunks must run in chain order"
-            )
-        tensor.copy_(group.mailbox.pop(key))
+        tensor.copy_(_loopback_pop(group, src, me, tag))
         return
     dist.recv(tensor, src=src, group=group)
 
 
+def state_take(like: torch.Tensor, src: int, group, dst: Optional[int] = None, tag: int = 0) -> torch.Tensor:
+    """The state rank `src` sent, as a tensor the caller owns (shaped like `like`).
+
+    In the loopback the parked copy itself changes hands, so a chunk's incoming state costs no
+    device copy beyond the one made when it was sent; over torch.distributed it is received into
+    a fresh buffer.  Either way the result can be kept for backward while `like` (the caller's KV
+    or DKV buffer) is overwritten with the outgoing state.
+    """
+    if isinstance(group, LoopbackGroup):
+        me = get_sequence_parallel_rank() if dst is None else dst
+        return _loopback_pop(group, src, me, tag)
+    t = torch.empty_like(like)
+    dist.recv(t, src=src, group=group)
+    return t
+
+
 def loopback_pending():
-    """(src, dst) pairs of states sent but not yet received (loopback mode only)."""
+    """(src, dst) pairs with states sent but not yet received (loopback mode only)."""
     grp = _st.sp_group
-    return sorted(grp.mailbox) if isinstance(grp, LoopbackGroup) else []
+    if not isinstance(grp, LoopbackGroup):
+        return []
+    return sorted({(src, dst) for (src, dst, _tag), q in grp.mailbox.items() if q})
 
 
 # ---------------------------------------------------------------- memory buffer

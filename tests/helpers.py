@@ -27,10 +27,13 @@ def oracle(inp, s, block=64, dtype=torch.float64):
 
 
 def check(got: dict, ref: dict, tol: float, names=NAMES, what=""):
-    errs = {}
+    """Asserts the parity bound on every (batch, head) slice of every output: the worst slice's
+    max|x - ref| / max|ref| must not exceed `tol`.  The whole-tensor figure goes into the message."""
+    errs, whole = {}, {}
     for name in names:
         if name in got and got[name] is not None:
             errs[name] = O.rel_err(got[name], ref[name])
+            whole[name] = O.rel_err_whole(got[name], ref[name])
     bad = {k_: v_ for k_, v_ in errs.items() if not (v_ <= tol)}
-    assert not bad, f"{what}: rel err over {tol}: {bad} (all: {errs})"
+    assert not bad, f"{what}: worst (b,h) slice over {tol}: {bad} (per-head: {errs}; whole tensor: {whole})"
     return errs

@@ -99,6 +99,24 @@ def test_null_and_workspace_errors_need_no_gpu(lib):
     assert rc == -5 and b"workspace" in lib.lasp_last_error()
 
 
+def test_alignment_and_device_errors_need_no_gpu(lib):
+    """A misaligned tensor or state pointer is LASP_E_ALIGN; a pointer HIP does not know as memory of
+    the current device is LASP_E_DEVICE.  Both are reported before anything is launched."""
+    ok, odd16, odd4 = ctypes.c_void_p(4096), ctypes.c_void_p(4096 + 8), ctypes.c_void_p(4096 + 2)
+    fwd = lambda q=ok, o=ok, kv=None, ws=ok: lib.lasp_chunk_fwd(q, ok, ok, ok, kv, None, o, ws, 1, 1, 1024, 128,
+                                                                 128, 1, 256, None)
+    assert fwd(q=odd16) == -6 and b"q" in lib.lasp_last_error() and b"16" in lib.lasp_last_error()
+    assert fwd(o=odd16) == -6 and b" o " in lib.lasp_last_error()
+    assert fwd(kv=odd4) == -6 and b"kv_in" in lib.lasp_last_error()
+    bwd = lambda dq=ok, dkv=None: lib.lasp_chunk_bwd(ok, ok, ok, ok, ok, None, dkv, dq, ok, ok, None, None, ok,
+                                                     1 << 30, 1, 1, 1024, 128, 128, 1, 256, None)
+    assert bwd(dq=odd16) == -6 and b"dq" in lib.lasp_last_error()
+    assert bwd(dkv=odd4) == -6 and b"dkv_in" in lib.lasp_last_error()
+    # well-aligned but not device memory (no GPU here, or a made-up address on a GPU box)
+    assert fwd() == -7 and b"q" in lib.lasp_last_error()
+    assert bwd() == -7
+
+
 def test_product_path_refuses_cpu_tensors(lib):
     import lasp_amd
     from lasp_amd import _abi

@@ -48,7 +48,7 @@ def _chain(op_name, q, k, v, do, s, chunks):
     e = v.shape[-1]
     step = n // chunks
     lasp_amd.initialize_lasp(1, chunks)
-    KV = torch.full((b, h, d, e), 7.0, dtype=torch.float64)   # garbage on entry: the operator zeroes it
+    KV = torch.full((b, h, d, e), 7.0, dtype=torch.float64)   # garbage on entry: the operator never reads it
     DKV = torch.full((b, h, d, e), -3.0, dtype=torch.float64)
     outs, leaves, kv_after = [], [], []
     for c in range(chunks):
@@ -64,11 +64,13 @@ def _chain(op_name, q, k, v, do, s, chunks):
         outs.append(o)
         leaves.append((qc, kc, vc))
         kv_after.append(KV.clone())
+    dkv_after = [None] * chunks
     for c in reversed(range(chunks)):
         outs[c].backward(do[:, :, c * step:(c + 1) * step])
+        dkv_after[c] = DKV.clone()
     assert lasp_amd.loopback_pending() == []
     cat = lambda i: torch.cat([l[i].grad for l in leaves], 2)
-    return torch.cat([o.detach() for o in outs], 2), cat(0), cat(1), cat(2), kv_after, DKV
+    return torch.cat([o.detach() for o in outs], 2), cat(0), cat(1), cat(2), kv_after, dkv_after
 
 
 @pytest.mark.parametrize("op_name", ["lasp_fuse", "lasp_fuse_parallel", "lasp_cache", "lasp_naive"])
@@ -76,17 +78,44 @@ def test_chain_choreography_equals_single_pass(op_name):
     q, k, v, do = _inputs(2, 3, 256, 16, 8, seed=1)
     s = O.slopes_alibi(3)
     ref = O.ref_chunked(q, k, v, s, do, dtype=torch.float64)
-    o, dq, dk, dv, kv_after, DKV = _chain(op_name, q, k, v, do, s, chunks=4)
+    o, dq, dk, dv, kv_after, dkv_after = _chain(op_name, q, k, v, do, s, chunks=4)
     tol = 1e-6 if op_name == "lasp_naive" else 1e-12  # lasp_naive allocates its own float32 state buffers
     for got, name in ((o, "o"), (dq, "dq"), (dk, "dk"), (dv, "dv")):
         assert O.rel_err(got, ref[name]) < tol, (op_name, name)
-    if op_name != "lasp_naive":  # lasp_naive owns its buffers
+    _, kv1 = O.ref_chunked_fwd(q[:, :, :64], k[:, :, :64], v[:, :, :64], s, None, 64, torch.float64)
+    _, kv3 = O.ref_chunked_fwd(q[:, :, :192], k[:, :, :192], v[:, :, :192], s, None, 64, torch.float64)
+    if op_name in ("lasp_fuse", "lasp_cache"):
         # the caller's KV holds KV_out of the chunk just run; after the last chunk, of the whole sequence
+        # (in-place update, lasp/lasp_fuse.py:126-127)
         assert O.rel_err(kv_after[-1], ref["kv_out"]) < 1e-12
-        _, kv1 = O.ref_chunked_fwd(q[:, :, :64], k[:, :, :64], v[:, :, :64], s, None, 64, torch.float64)
         assert O.rel_err(kv_after[0], kv1) < 1e-12
         # after the reversed chain the caller's DKV holds dL/dKV_in of the first chunk
-        assert O.rel_err(DKV, ref["dkv_out"]) < 1e-12
+        assert O.rel_err(dkv_after[0], ref["dkv_out"]) < 1e-12
+    elif op_name == "lasp_fuse_parallel":
+        # the caller's buffers are left holding the INCOMING states (lasp/lasp_fuse_parallel.py:1091-1101:
+        # KV is zeroed, received into, and the outgoing state is bound to a new tensor)
+        assert torch.count_nonzero(kv_after[0]) == 0
+        assert O.rel_err(kv_after[1], kv1) < 1e-12
+        assert O.rel_err(kv_after[-1], kv3) < 1e-12
+        assert torch.count_nonzero(dkv_after[-1]) == 0
+        # DKV entering chunk 0 = dL/dKV_out of chunk 0 = DKV_out of the chain over chunks 1..3
+        tail = O.ref_chunked(q[:, :, 64:], k[:, :, 64:], v[:, :, 64:], s, do[:, :, 64:], kv1, None,
+                             dtype=torch.float64)
+        assert O.rel_err(dkv_after[0], tail["dkv_out"]) < 1e-12
+
+
+@pytest.mark.parametrize("d", [192, 256])
+@pytest.mark.parametrize("op_name", ["lasp_fuse", "lasp_fuse_parallel", "lasp_cache", "lasp_naive"])
+def test_wide_heads_through_a_two_chunk_chain(op_name, d):
+    """d > 128 runs one chunk call per 128-wide feature slice, and every slice sends its own state to
+    the same neighbour: the loopback has to deliver them first-in first-out per slice."""
+    q, k, v, do = _inputs(1, 2, 128, d, 8, seed=7)
+    s = O.slopes_alibi(2)
+    ref = O.ref_chunked(q, k, v, s, do, dtype=torch.float64)
+    o, dq, dk, dv, _, _ = _chain(op_name, q, k, v, do, s, chunks=2)
+    tol = 1e-6 if op_name == "lasp_naive" else 1e-12
+    for got, name in ((o, "o"), (dq, "dq"), (dk, "dk"), (dv, "dv")):
+        assert O.rel_err(got, ref[name]) < tol, (op_name, d, name)
 
 
 def test_lightning_attn_and_wide_heads_are_sliced_and_summed():

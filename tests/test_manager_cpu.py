@@ -68,6 +68,30 @@ def test_loopback_mailbox_send_recv():
         spm.state_recv(out, 0, grp)
 
 
+
+def test_loopback_mailbox_is_first_in_first_out_per_pair_and_tag():
+    lasp_amd.initialize_lasp(1, 2)
+    grp = lasp_amd.get_sequence_parallel_group()
+    lasp_amd.set_sequence_parallel_rank(0)
+    first, second, tagged = torch.full((2,), 1.0), torch.full((2,), 2.0), torch.full((2,), 9.0)
+    spm.state_send(first, 1, grp)
+    spm.state_send(second, 1, grp)      # a second message to the same neighbour queues behind the first
+    spm.state_send(tagged, 1, grp, tag=1)
+    given = torch.full((2,), 5.0)
+    spm.state_send(given, 1, grp, tag=2, give=True)
+    assert lasp_amd.loopback_pending() == [(0, 1)]
+    lasp_amd.set_sequence_parallel_rank(1)
+    out = torch.empty(2)
+    spm.state_recv(out, 0, grp, tag=1)
+    assert torch.equal(out, tagged)
+    assert torch.equal(spm.state_take(out, 0, grp), first)
+    spm.state_recv(out, 0, grp)
+    assert torch.equal(out, second)
+    assert spm.state_take(out, 0, grp, tag=2).data_ptr() == given.data_ptr()   # handed over, not copied
+    assert lasp_amd.loopback_pending() == []
+    with pytest.raises(RuntimeError, match="nothing was sent"):
+        spm.state_take(out, 0, grp)
+
 def test_loopback_rejects_data_parallel():
     with pytest.raises(RuntimeError, match="sequence parallelism only"):
         lasp_amd.initialize_lasp(2, 2)

@@ -1,6 +1,7 @@
 """Parity of the HIP path (through the C ABI) against the CPU oracle.
 
-Error metric: max|x - ref| / max|ref| per output tensor, ref = fp64 oracle on the
+Error metric: max|x - ref| / max|ref| of every (batch, head) slice of every output tensor
+(the worst slice is held to the tolerance), ref = fp64 oracle on the
 same rounded inputs.  Tolerances: 1e-3 for fp32 I/O, 2e-2 for bf16 / fp16 I/O.
 """
 import pytest
