@@ -113,6 +113,28 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s,
                    void *stream);
 
 /*
+ * lasp_chunk_fwd without a workspace argument.  No counterpart in the reference: it is
+ * for callers that cannot allocate device memory around the call (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  Same computation and
+ * results as lasp_chunk_fwd; the segment states go to a scratch array of
+ * LASP_STATIC_SCRATCH_BYTES that is part of the library's code object (each GPU the
+ * library runs on holds its own copy until the process ends).  The call allocates and
+ * frees nothing, on the host or the device.
+ * Limit: b * h * n_seg states of 64 KiB (128 x 128 floats; d x e floats on the generic
+ * path) must fit, i.e. at most 512 states on the MFMA path -- the headline shape
+ * b=1 h=16 n=65536 with the default seg_len just fits; a larger call returns
+ * LASP_E_WORKSPACE (a longer seg_len lowers n_seg).
+ * All calls on one GPU share that GPU's scratch: two calls whose work overlaps in time
+ * on one GPU (different streams, or different threads) race on it.  The states are not
+ * returned, so a backward of the same chunk recomputes them (kv_seg_states = NULL).
+ */
+#define LASP_STATIC_SCRATCH_BYTES (32u << 20)
+int lasp_chunk_fwd_static(const void *q, const void *k, const void *v, const float *s,
+                          const float *kv_in, float *kv_out, void *o,
+                          int b, int h, int64_t n, int d, int e, int dtype, int seg_len,
+                          void *stream);
+
+/*
  * Backward (given dO and DKV_in = dL/dKV_out):
  *   dQ_i = sum_{j<=i} l^(i-j) (dO_i . v_j) k_j + l^i dO_i KV_in^T
  *   dK_j = sum_{i>=j} l^(i-j) (dO_i . v_j) q_i + l^(n-j) v_j DKV_in^T

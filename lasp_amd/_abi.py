@@ -58,6 +58,8 @@ def load() -> ctypes.CDLL:
     lib.lasp_kernel_path.argtypes = [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int]
     lib.lasp_chunk_fwd.restype = _c_int
     lib.lasp_chunk_fwd.argtypes = [_c_void_p] * 8 + [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
+    lib.lasp_chunk_fwd_static.restype = _c_int
+    lib.lasp_chunk_fwd_static.argtypes = [_c_void_p] * 7 + [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
     lib.lasp_chunk_bwd.restype = _c_int
     lib.lasp_chunk_bwd.argtypes = [_c_void_p] * 13 + [_c_size, _c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
     lib.lasp_profile_begin.restype = _c_int
@@ -202,6 +204,36 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     if rc:
         _raise(rc, "lasp_chunk_fwd")
     return o, states, seg_len
+
+
+STATIC_SCRATCH_BYTES = 32 << 20
+
+
+def chunk_fwd_static(q, k, v, s, o, kv_in=None, kv_out=None, seg_len: int = 0) -> None:
+    """Forward of one chunk into the caller's `o`, allocating nothing (lasp_chunk_fwd_static).
+
+    For code that must not allocate device memory around the call (graph capture, serving loops):
+    the segment states live in a scratch array inside the library, which limits the call to
+    STATIC_SCRATCH_BYTES of states (see `plan`) and means calls that overlap in time on one GPU
+    race.  Every tensor must already be contiguous and on the current device; s must be float32.
+    """
+    lib = load()
+    dev = _check_dev(q, k, v, o, s, kv_in, kv_out)
+    b, h, n, d, e = _shapes(q, k, v)
+    if o.shape != v.shape or o.dtype != q.dtype:
+        raise LaspError(f"o must match v: {tuple(o.shape)} {o.dtype} vs {tuple(v.shape)} {q.dtype}")
+    if s.dtype != torch.float32 or s.numel() != h:
+        raise LaspError(f"s must hold {h} float32 slopes, got {s.dtype} with {s.numel()} elements")
+    for name, t in (("q", q), ("k", k), ("v", v), ("o", o), ("s", s)):
+        if not t.is_contiguous():
+            raise LaspError(f"{name} must be contiguous (this call makes no copies)")
+    _check_state("kv_in", kv_in, b, h, d, e)
+    _check_state("kv_out", kv_out, b, h, d, e)
+    rc = lib.lasp_chunk_fwd_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
+                                   o.data_ptr(), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
+                                   torch.cuda.current_stream(dev).cuda_stream)
+    if rc:
+        _raise(rc, "lasp_chunk_fwd_static")
 
 
 def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_seg_states=None, seg_len: int = 0):

@@ -161,6 +161,44 @@ int check_device(const char *call, const void *q) {
   return 0;
 }
 
+// ---- segment-state scratch owned by the library (lasp_chunk_fwd_static) ------------------------
+// Lives in the code object: every device the library runs on holds its own copy, at its own
+// address, until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress -- the device address it returns (kept per device below) is what goes
+// into kernel arguments.
+static __device__ __align__(256) __attribute__((used)) float scratch[LASP_STATIC_SCRATCH_BYTES / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+static std::atomic<float *> g_scratch_ptr[kMaxDevices];  // zero-initialised: not looked up yet
+
+// Device address of `scratch` on the calling thread's current device (looked up once per device).
+int static_scratch(float **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("lasp_chunk_fwd_static: hipGetDevice failed: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    set_error("lasp_chunk_fwd_static: device ordinal %d is outside the supported range 0..%d", dev, kMaxDevices - 1);
+    return LASP_E_DEVICE;
+  }
+  float *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void *sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !sym) {
+      set_error("lasp_chunk_fwd_static: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+                hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : LASP_E_DEVICE;
+    }
+    p = (float *)sym;
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads store the same address
+  }
+  *out = p;
+  return 0;
+}
+
 size_t state_bytes_of(const Geom &g) {
   return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.sd * g.se;
 }
@@ -293,6 +331,29 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
     return LASP_E_WORKSPACE;
   }
   return chunk_fwd_impl("lasp_chunk_fwd", q, k, v, s, kv_in, kv_out, o, seg_states, g, dtype, stream);
+}
+
+int lasp_chunk_fwd_static(const void *q, const void *k, const void *v, const float *s, const float *kv_in,
+                          float *kv_out, void *o, int b, int h, int64_t n, int d, int e, int dtype,
+                          int seg_len, void *stream) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, seg_len, &g);
+  if (rc) return rc;
+  if (!q || !k || !v || !s || !o) {
+    set_error("lasp_chunk_fwd_static: q, k, v, s and o must not be NULL");
+    return LASP_E_NULL;
+  }
+  if (state_bytes_of(g) > (size_t)LASP_STATIC_SCRATCH_BYTES) {
+    set_error("lasp_chunk_fwd_static: the segment states of this call take %zu bytes (b*h*n_seg = %lld states), "
+              "the library's scratch holds %zu; pass a larger seg_len or use lasp_chunk_fwd with a workspace",
+              state_bytes_of(g), (long long)g.b * g.h * g.n_seg, (size_t)LASP_STATIC_SCRATCH_BYTES);
+    return LASP_E_WORKSPACE;
+  }
+  float *states = nullptr;
+  if ((rc = static_scratch(&states))) return rc;
+  // every state the kernels read from the scratch is one they wrote earlier in this same call, so
+  // nothing needs clearing between calls
+  return chunk_fwd_impl("lasp_chunk_fwd_static", q, k, v, s, kv_in, kv_out, o, states, g, dtype, stream);
 }
 
 int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, const void *d_o,

@@ -33,7 +33,7 @@ def _declared_functions():
 def test_header_declares_the_expected_entry_points():
     names = _declared_functions()
     for must in ("lasp_abi_version", "lasp_last_error", "lasp_plan", "lasp_kernel_path", "lasp_chunk_fwd",
-                 "lasp_chunk_bwd", "lasp_profile_begin", "lasp_profile_end"):
+                 "lasp_chunk_fwd_static", "lasp_chunk_bwd", "lasp_profile_begin", "lasp_profile_end"):
         assert must in names
 
 
@@ -115,6 +115,14 @@ def test_alignment_and_device_errors_need_no_gpu(lib):
     # well-aligned but not device memory (no GPU here, or a made-up address on a GPU box)
     assert fwd() == -7 and b"q" in lib.lasp_last_error()
     assert bwd() == -7
+
+
+def test_static_scratch_entry_rejects_oversized_calls_without_a_gpu(lib):
+    ok = ctypes.c_void_p(4096)
+    # b*h*n_seg = 16 * 64 states of 64 KiB = 64 MiB > the 32 MiB scratch
+    rc = lib.lasp_chunk_fwd_static(ok, ok, ok, ok, None, None, ok, 1, 16, 65536, 128, 128, 1, 1024, None)
+    assert rc == -5 and b"scratch holds" in lib.lasp_last_error()
+    assert lib.lasp_chunk_fwd_static(None, ok, ok, ok, None, None, ok, 1, 1, 64, 128, 128, 1, 0, None) == -1
 
 
 def test_product_path_refuses_cpu_tensors(lib):
