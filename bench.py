@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extras]
 
 One step = forward + backward of causal decayed linear attention through the
 public operator (lightning_attn + autograd) on the headline workload (TNL-1B head shape):
@@ -10,13 +10,28 @@ b=1, h=16, n=65536, d=e=128, bf16, Q/K/V/dO ~ N(0,1)/sqrt(d), slopes
 Prints ONE JSON line (metric = fwd+bwd tokens/s) that also carries
   roofline     -- la_bwd3, the dominant kernel, against the HBM roof: algorithmic
                   bytes per launch / its mean launch duration (HIP events around
-                  every launch, on the launch stream); roofline_fwd: the same for la_apply
+                  every launch, on the launch stream); roofline_fwd: the same for la_apply.
+                  `traffic` is read from the rocprofv3 counter summary under profiles/
+                  and is null when that summary was taken with another segment plan.
   cpu_baseline -- the CPU oracle (fp32 torch port of the same recurrence) timed on
-                  the host cores on one pass of the same workload.
+                  the host cores on a bounded number of passes of the same workload.
+  other_configs -- forward+backward times of the other benchmark configurations
+                  (0: fp32; 1: single pass and as 8 chunks through lasp_fuse and
+                  lasp_fuse_parallel; 3: one chunk with incoming KV; 4: 1M tokens as
+                  64 chunks), each with tokens/s and canonical TFLOP/s.
+
+Order of the run: the other configurations, then a settling phase (--settle-ms, default 150 ms
+of the headline step, untimed), then the W warm-up steps and the K timed steps.  The settling
+phase is there because the part answers every change of load with a power-management transient:
+for about 30 ms after these kernels start -- from idle or straight after other GPU work -- every
+kernel runs 5-30 % slower, back to back with no gaps between them, and then settles.  A training
+job sits in the settled regime, so that is what the timed steps measure; `settle_ms` is
+recorded in the output, and --settle-ms 0 shows the transient.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -31,13 +46,10 @@ FLOP_FWD_PER_TH = 98304        # 2Bd + 2Be + 4de at B=64, d=e=128
 FLOP_BWD_PER_TH = 245760       # 6Bd + 4Be + 10de
 BYTES_FWD_PER_TH = 1024        # read Q,K,V + write O, bf16
 BYTES_BWD_PER_TH = 1792        # read Q,K,V,dO + write dQ,dK,dV
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this workload
-# (profiles/pmc_hbm_bytes_config2.txt); FETCH_SIZE is scaled by 2.0 and WRITE_SIZE by 1.0, the
-# factors a plain 1 GiB device copy shows for the same counters.
-TRAFFIC_BWD3_BYTES = 2708338 * 1024   # 2 x 960 953 KiB fetched + 786 432 KiB written
-TRAFFIC_APPLY_BYTES = 1081509 * 1024  # 2 x 409 683 KiB fetched + 262 144 KiB written
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+MFMA_F32_PEAK_TFLOPS = 157.3
+HBM_PROFILE = os.path.join(ROOT, "profiles", "pmc_hbm_bytes_config2.txt")
 
 
 def slopes(h):
@@ -51,24 +63,59 @@ def make_inputs(device, n=N, seed=2):
     return [t.to(device) for t in (q, k, v, do)]
 
 
+def device_inputs(dev, b, h, n, d, dtype, seed, scale):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    return [(torch.randn(b, h, n, d, generator=g, device=dev) * scale).to(dtype) for _ in range(4)]
+
+
+def read_traffic_profile(path=HBM_PROFILE):
+    """HBM bytes per launch from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary.
+
+    The file states the segment plan it was taken with (`plan: seg_len=.. n_seg=..`), the scale factor of
+    each counter (from a plain device copy of known size) and one `traffic <kernel> fetch_kib=.. write_kib=..`
+    line per kernel.  Returns {"seg_len", "n_seg", "kernels": {name: bytes}} or None if there is no such file."""
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    plan = re.search(r"plan:\s*seg_len=(\d+)\s+n_seg=(\d+)", text)
+    scale = re.search(r"scale:\s*fetch=([0-9.]+)\s+write=([0-9.]+)", text)
+    if not plan or not scale:
+        return None
+    f_scale, w_scale = float(scale.group(1)), float(scale.group(2))
+    kernels = {}
+    for m in re.finditer(r"^traffic\s+(\S+)\s+fetch_kib=([0-9.]+)\s+write_kib=([0-9.]+)", text, flags=re.M):
+        kernels[m.group(1)] = int((float(m.group(2)) * f_scale + float(m.group(3)) * w_scale) * 1024)
+    return {"seg_len": int(plan.group(1)), "n_seg": int(plan.group(2)), "kernels": kernels}
+
+
+def cpu_cores():
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    return min(cores, os.cpu_count() or cores)
+
+
+def cpu_time_passes(fn, budget_s, max_passes):
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        passes += 1
+        if time.perf_counter() - t0 >= budget_s or passes >= max_passes:
+            break
+    return (time.perf_counter() - t0) / passes, passes
+
+
 def cpu_baseline():
-    """Oracle port (oracle/lasp_oracle.py: ref_chunked, fp32, block 64) on all host cores."""
+    """Oracle port (oracle/lasp_oracle.py: ref_chunked, fp32, block 64) on all host cores: the headline
+    workload for about 10 s, configurations 0 and 3 for a few seconds each."""
     from oracle import lasp_oracle as O
 
-    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
-    cores = min(cores, os.cpu_count() or cores)
+    cores = cpu_cores()
     torch.set_num_threads(cores)
     q, k, v, do = [t.float() for t in make_inputs("cpu")]
     s = slopes(H)
     O.ref_chunked(q[:, :, :1024], k[:, :, :1024], v[:, :, :1024], s, do[:, :, :1024])  # warm the thread pool
-    passes, t0 = 0, time.perf_counter()
-    while True:  # about 10 s of CPU work
-        O.ref_chunked(q, k, v, s, do, block=64, dtype=torch.float32)
-        passes += 1
-        if time.perf_counter() - t0 >= 10.0 or passes >= 16:
-            break
-    dt = (time.perf_counter() - t0) / passes
-    return {
+    dt, passes = cpu_time_passes(lambda: O.ref_chunked(q, k, v, s, do, block=64, dtype=torch.float32), 10.0, 16)
+    out = {
         "value": B * N / dt,
         "unit": "tokens/s",
         "cores": cores,
@@ -76,6 +123,169 @@ def cpu_baseline():
         "sample": f"{passes} fwd+bwd passes of the full workload (b={B} h={H} n={N} d={D}), fp32 torch, {dt:.2f} s each",
         "gflops": (FLOP_FWD_PER_TH + FLOP_BWD_PER_TH) * B * H * N / dt / 1e9,
     }
+    del q, k, v, do
+    g = torch.Generator().manual_seed(0)
+    q0, k0, v0, do0 = [torch.randn(2, 12, 2048, 128, generator=g) for _ in range(4)]
+    dt0, p0 = cpu_time_passes(lambda: O.ref_chunked(q0, k0, v0, slopes(12), do0, block=64, dtype=torch.float32), 3.0, 64)
+    g = torch.Generator().manual_seed(3)
+    q3, k3, v3, do3 = [torch.randn(1, 32, 16384, 128, generator=g) / D ** 0.5 for _ in range(4)]
+    kv3 = torch.randn(1, 32, 128, 128, generator=g) * 0.02
+    dt3, p3 = cpu_time_passes(lambda: O.ref_chunked(q3, k3, v3, slopes(32), do3, kv3, None, block=64,
+                                                    dtype=torch.float32), 4.0, 16)
+    out["other_configs"] = {
+        "config0_fp32": {"tokens_per_s": 2 * 2048 / dt0, "ms": dt0 * 1e3, "passes": p0},
+        "config3_chunk_with_kv_in": {"tokens_per_s": 16384 / dt3, "ms": dt3 * 1e3, "passes": p3},
+    }
+    return out
+
+
+def gpu_time(fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / iters * 1e3
+
+
+def rates(ms, b, h, n):
+    th = b * h * n
+    return {
+        "fwd_bwd_ms": ms,
+        "tokens_per_s": b * n / (ms * 1e-3),
+        "tflops": (FLOP_FWD_PER_TH + FLOP_BWD_PER_TH) * th / (ms * 1e-3) / 1e12,
+        "algorithmic_gbs": None,
+    }
+
+
+def with_bytes(r, b, h, n, elem_bytes):
+    r["algorithmic_gbs"] = (BYTES_FWD_PER_TH + BYTES_BWD_PER_TH) * (elem_bytes / 2) * b * h * n / (r["fwd_bwd_ms"] * 1e-3) / 1e9
+    return r
+
+
+def single_pass_step(lasp_amd, q, k, v, do, s):
+    def step():
+        q.grad = k.grad = v.grad = None
+        lasp_amd.lightning_attn(q, k, v, s).backward(do)
+
+    return step
+
+
+def chain_step(lasp_amd, op, parts, s, KV, DKV):
+    """Forward over the chunks in order, backward in reverse, through a public chunk operator with the
+    loopback standing in for the neighbouring ranks (one process plays every sequence-parallel rank)."""
+    chunks = len(parts)
+
+    def step():
+        outs = []
+        for c, (q, k, v, _do) in enumerate(parts):
+            q.grad = k.grad = v.grad = None
+            lasp_amd.set_sequence_parallel_rank(c)
+            outs.append(op(q, k, v, s, KV, DKV))
+        for c in reversed(range(chunks)):
+            lasp_amd.set_sequence_parallel_rank(c)
+            outs[c].backward(parts[c][3])
+
+    return step
+
+
+def split_chunks(tensors, chunks):
+    """Contiguous per-chunk leaves (each rank of a real run owns its chunk as a tensor of its own)."""
+    n = tensors[0].shape[2]
+    step = n // chunks
+    parts = []
+    for c in range(chunks):
+        sl = slice(c * step, (c + 1) * step)
+        q, k, v, do = [t[:, :, sl].contiguous() for t in tensors]
+        parts.append((q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True), do))
+    return parts
+
+
+def other_configs(dev):
+    """Forward+backward times of benchmark configurations 0, 1, 3 and 4 (synthetic inputs of their shapes)."""
+    import importlib
+
+    import lasp_amd
+
+    LF = importlib.import_module("lasp_amd.lasp_fuse")
+    out = {}
+
+    # configuration 0: fp32, b=2 h=12 n=2048, single pass
+    b, h, n = 2, 12, 2048
+    q, k, v, do = device_inputs(dev, b, h, n, D, torch.float32, 10, 1.0)
+    for t in (q, k, v):
+        t.requires_grad_(True)
+    r = with_bytes(rates(gpu_time(single_pass_step(lasp_amd, q, k, v, do, slopes(h).to(dev)), 50), b, h, n), b, h, n, 4)
+    r["frac_f32_mfma_peak"] = r["tflops"] / MFMA_F32_PEAK_TFLOPS
+    out["config0_fp32_single_pass"] = r
+    del q, k, v, do
+
+    # configuration 1: bf16, b=2 h=12 n=16384; single pass, then 8 chunks of 2048 with KV / DKV carry
+    b, h, n, chunks = 2, 12, 16384, 8
+    tensors = device_inputs(dev, b, h, n, D, torch.bfloat16, 11, 1.0)
+    s = slopes(h).to(dev)
+    q, k, v, do = tensors
+    ql, kl, vl = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    out["config1_single_pass"] = with_bytes(rates(gpu_time(single_pass_step(lasp_amd, ql, kl, vl, do, s), 30), b, h, n), b, h, n, 2)
+    del ql, kl, vl
+    parts = split_chunks(tensors, chunks)
+    KV = torch.empty(b, h, D, D, device=dev)
+    DKV = torch.empty_like(KV)
+    for name in ("lasp_fuse", "lasp_fuse_parallel"):
+        lasp_amd.destroy_parallel_groups()
+        lasp_amd.initialize_lasp(1, chunks)
+        try:
+            ms = gpu_time(chain_step(lasp_amd, getattr(lasp_amd, name), parts, s, KV, DKV), 20)
+        finally:
+            lasp_amd.destroy_parallel_groups()
+        r = with_bytes(rates(ms, b, h, n), b, h, n, 2)
+        r["chunks"] = chunks
+        r["vs_single_pass"] = ms / out["config1_single_pass"]["fwd_bwd_ms"]
+        out[f"config1_chain_{name}"] = r
+    del tensors, parts, q, k, v, do
+
+    # configuration 3: bf16, b=1 h=32, one chunk of 16384 with incoming KV ~ N(0, 0.02), DKV_in = 0,
+    # through lasp_fuse's launch shims (KV and DKV updated in place)
+    b, h, n = 1, 32, 16384
+    q, k, v, do = device_inputs(dev, b, h, n, D, torch.bfloat16, 13, D ** -0.5)
+    s = slopes(h).to(dev)
+    g = torch.Generator(device=dev).manual_seed(14)
+    kv_in = torch.randn(b, h, D, D, generator=g, device=dev) * 0.02
+    KV, DKV = torch.empty_like(kv_in), torch.empty_like(kv_in)
+
+    def step3():
+        KV.copy_(kv_in)
+        DKV.zero_()
+        LF.lasp_forward(q, k, v, s, KV)
+        LF.lasp_backward(q, k, v, s, do, kv_in, DKV)
+
+    out["config3_chunk_with_kv_in"] = with_bytes(rates(gpu_time(step3, 30), b, h, n), b, h, n, 2)
+    del q, k, v, do
+
+    # configuration 4a: bf16, b=1 h=16 n=1 048 576 as 64 chunks of 16384 through lasp_fuse
+    b, h, chunks, step = 1, 16, 64, 16384
+    n = chunks * step
+    s = slopes(h).to(dev)
+    parts = []
+    for c in range(chunks):
+        q, k, v, do = device_inputs(dev, b, h, step, D, torch.bfloat16, 1000 + c, D ** -0.5)
+        parts.append((q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True), do))
+    KV = torch.empty(b, h, D, D, device=dev)
+    DKV = torch.empty_like(KV)
+    lasp_amd.destroy_parallel_groups()
+    lasp_amd.initialize_lasp(1, chunks)
+    try:
+        ms = gpu_time(chain_step(lasp_amd, lasp_amd.lasp_fuse, parts, s, KV, DKV), 3, warm=1)
+    finally:
+        lasp_amd.destroy_parallel_groups()
+    r = with_bytes(rates(ms, b, h, n), b, h, n, 2)
+    r["chunks"] = chunks
+    out["config4a_1m_tokens_chain_lasp_fuse"] = r
+    del parts
+    torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -84,6 +294,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (profiling runs)")
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="run the headline step untimed for this long before the warm-up steps (see the module docstring)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -97,7 +310,11 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    # the headline inputs are made (on the host, seeded) before anything runs on the GPU, so that no idle
+    # stretch separates the other configurations from the headline's warm-up
     q, k, v, do = make_inputs(dev)
+    extras = None if args.no_extras else other_configs(dev)
     q.requires_grad_(True)
     k.requires_grad_(True)
     v.requires_grad_(True)
@@ -112,15 +329,19 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    def step():
-        q.grad = k.grad = v.grad = None
-        o = lasp_amd.lightning_attn(q, k, v, s)
-        o.backward(do)
+    step = single_pass_step(lasp_amd, q, k, v, do, s)
 
     def fwd_only():
         with torch.no_grad():
             lasp_amd.lightning_attn(q, k, v, s)
 
+    settle_steps = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < args.settle_ms:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        settle_steps += 10
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -146,14 +367,20 @@ def main():
         step()
     prof = _abi.profile_end()
     th = B * H * N
+    kernel_sum_ms = sum(ms for ms, cnt in prof.values()) / args.steps
 
-    def roof(kernel, cls, alg_bytes, traffic):
+    profile = read_traffic_profile()
+    same_plan = profile is not None and (profile["seg_len"], profile["n_seg"]) == (seg_len, n_seg)
+
+    def roof(kernel, cls, alg_bytes):
         ms, cnt = prof[cls]
         avg_ms = ms / max(cnt, 1)
         achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
         return {
             "kernel": kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": profile["kernels"].get(kernel) if same_plan else None,
+            "traffic_source": os.path.relpath(HBM_PROFILE, ROOT) if same_plan else None,
             "algorithmic_bytes_per_launch": alg_bytes, "avg_launch_ms": avg_ms, "launches": cnt,
         }
 
@@ -167,6 +394,8 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
+        "settle_steps": settle_steps,
         "ms_per_step": ms_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -184,12 +413,16 @@ def main():
         "fwd_bwd_tflops": tflops,
         "frac_bf16_mfma_peak": tflops / MFMA_BF16_PEAK_TFLOPS,
         "step_algorithmic_gbs": (BYTES_FWD_PER_TH + BYTES_BWD_PER_TH) * th / (ms_step * 1e-3) / 1e9,
+        "frac_hbm_peak_step": (BYTES_FWD_PER_TH + BYTES_BWD_PER_TH) * th / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": {name: {"total_ms": ms, "launches": cnt} for name, (ms, cnt) in prof.items() if cnt},
+        "kernel_sum_ms_per_step": kernel_sum_ms,
         # dominant kernel: la_bwd3 (one launch = the whole backward sweep: reads Q,K,V,dO, writes dQ,dK,dV)
-        "roofline": roof("la_bwd3", "bwd3", BYTES_BWD_PER_TH * th, TRAFFIC_BWD3_BYTES),
+        "roofline": roof("la_bwd3", "bwd3", BYTES_BWD_PER_TH * th),
         # second kernel: la_apply (one launch = the forward sweep: reads Q,K,V, writes O)
-        "roofline_fwd": roof("la_apply", "apply", BYTES_FWD_PER_TH * th, TRAFFIC_APPLY_BYTES),
+        "roofline_fwd": roof("la_apply", "apply", BYTES_FWD_PER_TH * th),
     }
+    if extras is not None:
+        out["other_configs"] = extras
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out), flush=True)

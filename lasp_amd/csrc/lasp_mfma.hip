@@ -93,6 +93,18 @@ struct ElemF16 {
   }
 };
 
+// A pointer that is the same for every lane, moved to scalar registers: loads through it then take
+// the form scalar base + 32-bit lane offset + immediate, instead of a 64-bit address per lane that
+// the loop optimiser would otherwise carry (and increment) in vector registers.  The result is
+// typed as a global-memory pointer, which the round trip through integers would otherwise lose.
+typedef const __attribute__((address_space(1))) char *gmem_ptr;
+__device__ __forceinline__ gmem_ptr uniform_ptr(const char *p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (gmem_ptr)(((uint64_t)hi << 32) | lo);
+}
+
 __device__ __forceinline__ u32x4 lds16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
 // element x (0..7) of a 16-byte group of 16-bit elements, widened to fp32
@@ -194,6 +206,21 @@ __device__ __forceinline__ u32x4 load_row_pieces(const char *tile, int64_t row_b
   const u32x2 zero = {0u, 0u};
   const u32x2 lo = (row_ok && ok.lo) ? *reinterpret_cast<const u32x2 *>(p + lane_off) : zero;
   const u32x2 hi = (row_ok && ok.hi) ? *reinterpret_cast<const u32x2 *>(p + lane_off + 16) : zero;
+  u32x4 r;
+  r.x = lo.x;
+  r.y = lo.y;
+  r.z = hi.x;
+  r.w = hi.y;
+  return r;
+}
+// the same through a scalar block pointer (see uniform_ptr)
+__device__ __forceinline__ u32x4 load_row_pieces(gmem_ptr tile, int row_bytes, uint32_t lane_off, PieceMask ok,
+                                                 bool row_ok) {
+  typedef const __attribute__((address_space(1))) u32x2 *gmem_u32x2;
+  gmem_ptr p = tile + row_bytes;
+  const u32x2 zero = {0u, 0u};
+  const u32x2 lo = (row_ok && ok.lo) ? *reinterpret_cast<gmem_u32x2>(p + lane_off) : zero;
+  const u32x2 hi = (row_ok && ok.hi) ? *reinterpret_cast<gmem_u32x2>(p + lane_off + 16) : zero;
   u32x4 r;
   r.x = lo.x;
   r.y = lo.y;
@@ -543,26 +570,49 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
 // A segment's own state:  causal  sum_b l^(L-b) y_b^T z_b ;  anti-causal  sum_b l^b y_b^T z_b
 // (b from the segment start, L its length), written token-free as 128 x 128 fp32.  Y rows hold
 // g.d features and Z rows g.e (M_NARROW; 128 otherwise).
+//
+// Blocks whose every token carries a weight below 2^-SKIP_LOG2 are neither read nor multiplied:
+// with slope s a token that lies x tokens from the segment's far end weighs exp(-s x), so a
+// fast-decaying head only needs the last (causal) or first (anti-causal) SKIP_LOG2 ln2 / s tokens
+// of each segment.  What is dropped is below 2^-64 of a full-weight term, far under the fp32
+// rounding (2^-24) of the sum it would be added to.  s = 0 skips nothing.
+//
+// That leaves the workgroups unevenly loaded -- those of slow-decaying heads still read whole
+// segments -- so one workgroup has to be able to pull more than an even share of the memory
+// bandwidth.  512 threads (8 waves, one workgroup per CU): threads 0-255 fetch the Y tile, 256-511
+// the Z tile, each keeping STATE_DEPTH blocks in flight in registers (16 registers per block) on
+// top of the two LDS buffers; wave (wc, rh) owns rows [64 rh, 64 rh + 64) x columns
+// [32 wc, 32 wc + 32) of the state as two accumulator tiles.
+constexpr float SKIP_LOG2 = 64.f;
+constexpr int STATE_THREADS = 512;
+constexpr int STATE_DEPTH = 2;  // blocks in flight per thread in registers (even); deeper measured slower:
+                                // the repeated loads at the end of a walk cost more than the depth gains
+
 template <class E, bool REV, int MODE>
-__global__ void __launch_bounds__(NTHR, 2)
+__global__ void __launch_bounds__(STATE_THREADS, 1)
 la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
+  constexpr int D = STATE_DEPTH;
   __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
+  const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
+  const int wc = w8 & 3, rh = w8 >> 2;                      // column block and row half of this wave's tiles
+  const bool zgrp = w8 >= 4;                                // this wave fetches Z (else Y)
   const int c = lane & 31, hh = lane >> 5;
-  const LoaderRole yr = yz_role(tid);
+  const LoaderRole yr = yz_role(tid & 255);
 
-  const SegWork sw = seg_work(g, (int)blockIdx.x);
+  // slow-decaying heads (the later ones in the usual slope schedules) have the most to read: first
+  const int n_items = g.b * g.h * g.n_seg;
+  const SegWork sw = seg_work(g, n_items - 1 - (int)blockIdx.x);
   if (sw.seg == skip_seg) return;  // the scan's final segment feeds only the outgoing carry
   const float sl = S[sw.bh % g.h] * LOG2E;
   const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;
   const int yw = NARROW ? g.d : F, zw = NARROW ? g.e : F;  // row widths in elements
-  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * yw);
-  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * zw);
-  const int yu = yw / 4, zu = zw / 4;  // 8-byte units per row
+  const int tw = zgrp ? zw : yw;                           // of the tile this thread fetches
+  const char *Tg = reinterpret_cast<const char *>(zgrp ? Z + row0 * zw : Y + row0 * yw);
+  const int tu = tw / 4;  // 8-byte units per row
 
   const float blockdec = decay(sl, (float)BLK);
   float kdec[4];
@@ -572,84 +622,117 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
     kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
   }
 
-  floatx16 st[4];
+  // blocks lo..hi of the segment are processed (uniform across the workgroup)
+  int lo = 0, hi = sw.nblk - 1;
+  if (sl > 0.f) {
+    const float keep = SKIP_LOG2 / sl;  // tokens whose weight is at least 2^-SKIP_LOG2
+    if (!REV) {
+      // the last token of block t lies (tokens - 64 t - 63) tokens before the segment end
+      const float x = ((float)((sw.nblk - 1) * BLK + sw.tail) - 63.f - keep) * (1.f / BLK);
+      if (x > 0.f) lo = min((int)ceilf(x), hi);
+    } else {
+      // the first token of block t lies 64 t tokens after the segment start
+      const float x = keep * (1.f / BLK);
+      if (x < (float)hi) hi = (int)x;
+    }
+  }
+  // the float arithmetic above ran on the vector unit; put the (uniform) results back in scalar
+  // registers so that the block addresses stay scalar
+  lo = __builtin_amdgcn_readfirstlane(lo);
+  hi = __builtin_amdgcn_readfirstlane(hi);
+  const int cnt = hi - lo + 1;
+
+  floatx16 st[2];
 #pragma unroll
-  for (int T = 0; T < 4; ++T)
+  for (int T = 0; T < 2; ++T)
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
 
   // A partial block (the end of a ragged chunk) reads its missing rows as zeros; going
   // forwards it is the last block, and its tokens sit `len - b` (not 64 - b) before the
   // segment end.
-  u32x4 ny[4], nz[4];
-  const uint32_t y_off = lane_offset(yr, 4 * yr.rowq, yu), z_off = lane_offset(yr, 4 * yr.rowq, zu);
-  const PieceMask y_ok = piece_mask(yr, yu), z_ok = piece_mask(yr, zu);
-  auto issue_loads = [&](int blk) __attribute__((always_inline)) {
+  const uint32_t t_off = lane_offset(yr, 4 * yr.rowq, tu);
+  const PieceMask t_ok = piece_mask(yr, tu);
+  // every address is a workgroup-uniform row pointer plus one per-thread 32-bit offset
+  auto issue_loads = [&](u32x4 (&nt)[4], int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    const int64_t yblk = (int64_t)blk * BLK * yu * 8, zblk = (int64_t)blk * BLK * zu * 8;  // bytes
+    const gmem_ptr tblk = uniform_ptr(Tg + (int64_t)blk * BLK * tu * 8);
+    const PieceMask all = {true, true};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const bool row_ok = 4 * yr.rowq + r < len;
-      if (!NARROW) {
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-        const int64_t row = (int64_t)blk * BLK + 4 * yr.rowq + r;
-        ny[r] = (!RAGGED || row_ok) ? load_row_pieces(Yg + row * 32, yr) : zero;
-        nz[r] = (!RAGGED || row_ok) ? load_row_pieces(Zg + row * 32, yr) : zero;
-      } else {
-        ny[r] = load_row_pieces(reinterpret_cast<const char *>(Yg), yblk + (int64_t)r * yu * 8, y_off, y_ok, row_ok);
-        nz[r] = load_row_pieces(reinterpret_cast<const char *>(Zg), zblk + (int64_t)r * zu * 8, z_off, z_ok, row_ok);
-      }
+      const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
+      nt[r] = load_row_pieces(tblk, r * tu * 8, t_off, NARROW ? t_ok : all, row_ok);
     }
   };
-  auto fill_lds = [&](int buf, int blk) __attribute__((always_inline)) {
+  auto fill_lds = [&](int buf, const u32x4 (&nt)[4], int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    if (RAGGED && !REV && len != BLK) {
+    if (zgrp) {
+      store_transposed<E, false>(smem[buf] + F * LDT, nt, yr, kdec);
+    } else if (RAGGED && !REV && len != BLK) {
       float kd[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
-      store_transposed<E, true>(smem[buf], ny, yr, kd);
+      store_transposed<E, true>(smem[buf], nt, yr, kd);
     } else {
-      store_transposed<E, true>(smem[buf], ny, yr, kdec);
+      store_transposed<E, true>(smem[buf], nt, yr, kdec);
     }
-    store_transposed<E, false>(smem[buf] + F * LDT, nz, yr, kdec);
   };
-
-  const int first = REV ? sw.nblk - 1 : 0;
-  const int step = REV ? -1 : 1;
-  issue_loads(first);
-  fill_lds(0, first);
-  __syncthreads();
-  for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
-    const bool more = it + 1 < sw.nblk;
-    if (more) issue_loads(blk + step);
+  // M_NARROW: columns past the width of Z stay zero, as do rows past Y's
+  const bool wave_active = !NARROW || (32 * wc < g.e && (rh == 0 || g.d > 64));
+  auto accumulate = [&](int buf, int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
     const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
-    const char *yt = smem[it & 1];
+    const char *yt = smem[buf];
     const char *zt = yt + F * LDT;
-    if (!NARROW || 32 * w < g.e) {  // M_NARROW: columns past the width of Z stay zero, as do rows past Y's
+    if (wave_active) {
       u32x4 zf[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * w + c, 2 * u + hh));
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * wc + c, 2 * u + hh));
 #pragma unroll
-      for (int T = 0; T < 4; ++T) {
-        if (NARROW && T >= 2 && g.d <= 64) continue;
+      for (int T = 0; T < 2; ++T) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          st[T] = E::mfma(lds16(yt + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
+          st[T] = E::mfma(lds16(yt + tr_off(64 * rh + 32 * T + c, 2 * u + hh)), zf[u], st[T]);
       }
     }
-    if (more) fill_lds((it + 1) & 1, blk + step);
-    __syncthreads();
+  };
+
+  // Block i of the walk (0 <= i < cnt) travels through register set i mod D.  Loads and LDS fills
+  // past the end of the walk are not skipped but repeat its last block (served by the cache, never
+  // used): with the same number of loads in flight on every path, the wait before a fill covers
+  // exactly the oldest register set.
+  const int first = REV ? hi : lo;
+  const int step = REV ? -1 : 1;
+  auto block_of = [&](int i) __attribute__((always_inline)) { return first + min(i, cnt - 1) * step; };
+  u32x4 set[D][4];
+#pragma unroll
+  for (int k = 0; k < D; ++k) issue_loads(set[k], block_of(k));
+  fill_lds(0, set[0], block_of(0));
+  issue_loads(set[0], block_of(D));
+  __syncthreads();
+  for (int i = 0; i < cnt; i += D) {
+#pragma unroll
+    for (int k = 0; k < D; ++k) {  // D is even: LDS buffer (i + k) & 1 == k & 1
+      if (i + k >= cnt) break;
+      accumulate(k & 1, block_of(i + k));
+      __builtin_amdgcn_sched_barrier(0);
+      fill_lds((k + 1) & 1, set[(k + 1) % D], block_of(i + k + 1));
+      __builtin_amdgcn_sched_barrier(0);
+      issue_loads(set[(k + 1) % D], block_of(i + k + 1 + D));
+      __syncthreads();
+    }
   }
 
-  float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
+  {
+    float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
 #pragma unroll
-  for (int T = 0; T < 4; ++T)
+    for (int T = 0; T < 2; ++T)
 #pragma unroll
-    for (int r = 0; r < 16; ++r)
-      sp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
+      for (int r = 0; r < 16; ++r)
+        sp[(64 * rh + 32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * wc + c] = st[T][r];
+  }
 }
 
 template <class E, bool REV, bool TRANS, int MODE>
@@ -688,7 +771,7 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
   ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, MODE><<<grid, NTHR, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
+  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
                                                       skip_seg);
   return (int)hipGetLastError();
 }

@@ -1,4 +1,9 @@
-"""lasp_fuse: per-rank chunk with KV in/out, states recomputed in backward (lasp/lasp_fuse.py)."""
+"""lasp_fuse: per-rank chunk with KV state in and out (lasp/lasp_fuse.py).
+
+The reference's backward re-runs the kv recurrence (lasp/lasp_fuse.py:237-260).  Here the forward
+leaves the state entering each segment in a workspace anyway, so the operator keeps it for backward
+(64 KiB per (b, h, segment)) instead of re-reading K and V to rebuild it; the launch shims below
+recompute, as they have no place to keep it."""
 import torch
 
 from . import _abi
@@ -31,7 +36,7 @@ class LaspFuse(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, s, KV, DKV):
-        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, False, False)
+        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, True, False)
 
     @staticmethod
     def backward(ctx, do):
@@ -45,4 +50,4 @@ def lasp_fuse(q, k, v, ed, KV, DKV):
     """KV, DKV: float32 (b, h, d, e) scratch owned by the caller; KV is left holding KV_out."""
     if q.shape[-1] <= 128:
         return lasp_fuse_(q, k, v, ed, KV, DKV)
-    return run_sliced(q, k, v, ed, KV, DKV, False, False)
+    return run_sliced(q, k, v, ed, KV, DKV, True, False)

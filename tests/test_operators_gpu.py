@@ -202,3 +202,52 @@ def test_launch_shims_against_oracle(gpu_device, dtype, e):
     torch.cuda.synchronize()
     assert torch.equal(KV, inp["kv"]) and torch.equal(DKV, inp["dkv"])
     check(dict(o=o, kv_out=KV_out, dq=dq, dk=dk, dv=dv, dkv_out=DKV_out), ref, TOL[dtype], what="lasp_fuse_parallel shims")
+
+
+def test_naive_and_cache_launch_shims_against_oracle(gpu_device):
+    """lasp_naive.lasp_forward / lasp_backward and the lasp_cache pair: the chunk with no incoming state plus the
+    chunk's own kv / dkv contributions in q.dtype (lasp/lasp_naive.py:429-538, lasp/lasp_cache.py:427-536).
+    Combining them the way LaspNaive does (torch matmuls for the incoming-state terms, :560-565, :604-614)
+    must reproduce the oracle with states."""
+    import importlib
+
+    from tests.helpers import check, oracle
+
+    LN = importlib.import_module("lasp_amd.lasp_naive")
+    LC = importlib.import_module("lasp_amd.lasp_cache")
+    dev = gpu_device
+    b, h, n, d, e = 1, 4, 512, 128, 64
+    s = O.slopes_baseline(h)
+    inp = make_inputs(b, h, n, d, e, torch.bfloat16, seed=33, scale=d ** -0.5, state=True, device=dev)
+    q, k, v, do, sd = inp["q"], inp["k"], inp["v"], inp["do"], s.to(dev)
+    stateless = dict(inp, kv=None, dkv=None)
+    ref0 = oracle(stateless, s)
+
+    kv = torch.empty(b, h, d, e, dtype=torch.bfloat16, device=dev)
+    o = LN.lasp_forward(q, k, v, sd, kv)
+    dq, dk, dv, none, dkv = LN.lasp_backward(q, k, v, sd, do)
+    o2, kv2 = LC.lasp_forward(q, k, v, sd)
+    dq2, dk2, dv2, none2, dkv2 = LC.lasp_backward(q, k, v, sd, do)
+    torch.cuda.synchronize()
+    assert none is None and none2 is None and kv.dtype == dkv.dtype == kv2.dtype == torch.bfloat16
+    for a_, b_ in ((o, o2), (kv, kv2), (dq, dq2), (dk, dk2), (dv, dv2), (dkv, dkv2)):
+        assert torch.equal(a_, b_)
+    check(dict(o=o, kv_out=kv, dq=dq, dk=dk, dv=dv, dkv_out=dkv), ref0, 2e-2, what="stateless shims")
+
+    # the reference's torch epilogue for the incoming-state terms, in fp32
+    ref = oracle(inp, s)
+    pos = torch.arange(n, device=dev, dtype=torch.float32)
+    sv = sd.reshape(1, h, 1, 1)
+    q_decay = torch.exp(-sv * pos.reshape(1, 1, n, 1))
+    k_decay = torch.exp(-sv * (n - pos).reshape(1, 1, n, 1))
+    block_decay = torch.exp(-sv * n)
+    KV, DKV = inp["kv"], inp["dkv"]
+    full = dict(
+        o=o.float() + torch.matmul(q.float() * q_decay, KV),
+        kv_out=block_decay * KV + kv.float(),
+        dq=dq.float() + torch.matmul(do.float(), KV.transpose(-1, -2)) * q_decay,
+        dk=dk.float() + torch.matmul(v.float(), DKV.transpose(-1, -2)) * k_decay,
+        dv=dv.float() + torch.matmul(k.float() * k_decay, DKV),
+        dkv_out=block_decay * DKV + dkv.float(),
+    )
+    check(full, ref, 2e-2, what="shims + torch epilogue")
