@@ -335,44 +335,24 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
                  z_off = lane_offset(yr, 4 * yr.rowq, zu);
   const PieceMask x_ok = piece_mask(xr, xu), y_ok = piece_mask(yr, xu), z_ok = piece_mask(yr, zu);
   // a partial block (the end of a ragged chunk) reads its missing rows as zeros
+  // every address is a workgroup-uniform block pointer (scalar registers) plus a per-thread 32-bit
+  // offset and an immediate; rows past a partial block's end and pieces past a narrow row's width
+  // read as zeros
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    if (!NARROW) {
-      const int64_t off = (int64_t)blk * (BLK * F / 4);  // in 8-byte units (32 per row)
-      if (!RAGGED || len == BLK) {
+    const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * xu * 8);
+    const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * xu * 8);
+    const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * zu * 8);
+    const PieceMask all = {true, true};
 #pragma unroll
-        for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(Xg + off + (xr.rowq + 16 * it) * 32, xr);
+    for (int it = 0; it < 4; ++it)
+      nx[it] = load_row_pieces(xblk, 16 * it * xu * 8, x_off, NARROW ? x_ok : all,
+                               !RAGGED || xr.rowq + 16 * it < len);
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          ny[r] = load_row_pieces(Yg + off + (4 * yr.rowq + r) * 32, yr);
-          nz[r] = load_row_pieces(Zg + off + (4 * yr.rowq + r) * 32, yr);
-        }
-      } else {
-        const u32x4 zero = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int it = 0; it < 4; ++it) {
-          const int row = xr.rowq + 16 * it;
-          nx[it] = row < len ? load_row_pieces(Xg + off + row * 32, xr) : zero;
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = 4 * yr.rowq + r;
-          ny[r] = row < len ? load_row_pieces(Yg + off + row * 32, yr) : zero;
-          nz[r] = row < len ? load_row_pieces(Zg + off + row * 32, yr) : zero;
-        }
-      }
-    } else {
-      const int64_t xblk = (int64_t)blk * BLK * xu * 8, zblk = (int64_t)blk * BLK * zu * 8;  // bytes
-#pragma unroll
-      for (int it = 0; it < 4; ++it)
-        nx[it] = load_row_pieces(reinterpret_cast<const char *>(Xg), xblk + (int64_t)(16 * it) * xu * 8, x_off,
-                                 x_ok, xr.rowq + 16 * it < len);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const bool row_ok = 4 * yr.rowq + r < len;
-        ny[r] = load_row_pieces(reinterpret_cast<const char *>(Yg), xblk + (int64_t)r * xu * 8, y_off, y_ok, row_ok);
-        nz[r] = load_row_pieces(reinterpret_cast<const char *>(Zg), zblk + (int64_t)r * zu * 8, z_off, z_ok, row_ok);
-      }
+    for (int r = 0; r < 4; ++r) {
+      const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
+      ny[r] = load_row_pieces(yblk, r * xu * 8, y_off, NARROW ? y_ok : all, row_ok);
+      nz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
     }
   };
   auto fill_lds = [&]() __attribute__((always_inline)) {
@@ -479,9 +459,14 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
     // (3) intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
     //     (token step outermost, so that consecutive MFMAs write different accumulators)
     if (wave_active) {
+      // The swizzled addresses of the feature-major tiles are recomputed for every block (a few
+      // integer operations each) rather than held in some twenty registers for the whole sweep:
+      // the opaque copy of the lane's column keeps the compiler from hoisting them.
+      int cc = c;
+      asm volatile("" : "+v"(cc));
       u32x4 zf[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + c, 2 * u + hh));
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + cc, 2 * u + hh));
       __builtin_amdgcn_s_setprio(1);
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -500,7 +485,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 #pragma unroll
         for (int T = 0; T < 4; ++T)
           if (!NARROW || T < 2 || fa > 64)  // state rows past the width of Y stay zero
-            st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + c, 2 * u + hh)), zf[u], st[T]);
+            st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + cc, 2 * u + hh)), zf[u], st[T]);
 
       __builtin_amdgcn_s_setprio(0);
     }
