@@ -74,6 +74,13 @@ extern "C" {
 #define LASP_PATH_MFMA 1    /* MFMA kernels, any n (a ragged tail is masked): bf16 / fp16 with d and e
                                multiples of 8 (rows narrower than 128 are read zero-extended), fp32 with
                                d = e = 128 */
+#define LASP_PATH_MFMA_FUSED 2 /* short chunks of the 16-bit MFMA shapes called with seg_len = 0 (n <= 2048
+                               and few enough segments that rebuilding a segment's incoming state from
+                               the blocks before it is cheaper than a pre-pass and a scan): one launch
+                               per direction; NO workspace is read or written (seg_states,
+                               kv_seg_states and workspace may be NULL and are ignored) and the forward
+                               leaves no segment states behind.  An explicit seg_len selects
+                               LASP_PATH_MFMA instead. */
 
 int lasp_abi_version(void);
 
@@ -94,7 +101,8 @@ const char *lasp_last_error(void);
 int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0,
               int *seg_len, int *n_seg, size_t *state_bytes);
 
-/* LASP_PATH_* for this shape, or a negative LASP_E_* if it is unsupported. */
+/* LASP_PATH_* for this shape under the default plan (seg_len = 0), or a negative LASP_E_* if it is
+ * unsupported. */
 int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype);
 
 /*
@@ -164,12 +172,13 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
  * any thread while it is open (each claims its slot atomically), begin and end
  * are called by one thread.
  */
-#define LASP_KERNEL_CLASSES 5
+#define LASP_KERNEL_CLASSES 6
 #define LASP_KC_APPLY 0   /* la_apply: the block sweep producing O */
 #define LASP_KC_STATE 1   /* la_seg_state: per-segment state pre-pass */
 #define LASP_KC_SCAN 2    /* decayed scan over segment states */
 #define LASP_KC_GENERIC 3 /* any kernel of the generic fp32-FMA family */
 #define LASP_KC_BWD3 4    /* la_bwd3: dQ, dK and dV block sweeps in one launch */
+#define LASP_KC_FUSED 5   /* la_fused_fwd / la_fused_bwd: a short chunk in one launch */
 int lasp_profile_begin(int max_launches);
 int lasp_profile_end(double *ms_per_class, int *launches_per_class);
 

@@ -20,7 +20,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "liblasp_hi
 _lib = None
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
-PATH_GENERIC, PATH_MFMA = 0, 1
+PATH_GENERIC, PATH_MFMA, PATH_MFMA_FUSED = 0, 1, 2
 
 _c_void_p = ctypes.c_void_p
 _c_int = ctypes.c_int
@@ -114,14 +114,16 @@ def plan(b: int, h: int, n: int, d: int, e: int, dtype: torch.dtype, seg_len: in
     return sl.value, ns.value, sb.value
 
 
+@functools.lru_cache(maxsize=256)
 def kernel_path(b, h, n, d, e, dtype) -> int:
+    """PATH_* a shape runs on when it is given to the library with the default plan (seg_len = 0)."""
     rc = load().lasp_kernel_path(b, h, n, d, e, DTYPE_CODE[dtype])
     if rc < 0:
         _raise(rc, "lasp_kernel_path")
     return rc
 
 
-KERNEL_CLASSES = ("apply", "state", "scan", "generic", "bwd3")
+KERNEL_CLASSES = ("apply", "state", "scan", "generic", "bwd3", "fused")
 
 
 def profile_begin(max_launches: int = 4096) -> None:
@@ -191,11 +193,15 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     s = _slopes(s, h, dev)
     _check_state("kv_in", kv_in, b, h, d, e)
     _check_state("kv_out", kv_out, b, h, d, e)
-    seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
+    # short chunks under the default plan run as one launch that needs no workspace and leaves no
+    # segment states; seg_len stays 0 so that the backward makes the same choice
+    fused = seg_len == 0 and kernel_path(b, h, n, d, e, q.dtype) == PATH_MFMA_FUSED
+    if not fused:
+        seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
     with _on_device(dev):
         o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
         states = None
-        if n_seg > 1 or kv_in is not None or kv_out is not None:
+        if not fused and (n_seg > 1 or kv_in is not None or kv_out is not None):
             # the library decides how a state is stored (d x e, or zero-extended to 128 x 128)
             states = torch.empty((b, h, n_seg, state_bytes // (4 * b * h * n_seg)), dtype=torch.float32, device=dev)
         rc = lib.lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
@@ -248,7 +254,11 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
     _check_state("kv_in", kv_in, b, h, d, e)
     _check_state("dkv_in", dkv_in, b, h, d, e)
     _check_state("dkv_out", dkv_out, b, h, d, e)
-    seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
+    fused = seg_len == 0 and kernel_path(b, h, n, d, e, q.dtype) == PATH_MFMA_FUSED
+    if fused:
+        n_seg, state_bytes, kv_seg_states = 1, 0, None  # one launch, no workspace, no use for cached states
+    else:
+        seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
     if kv_seg_states is not None:
         if (kv_seg_states.dtype != torch.float32 or kv_seg_states.numel() * 4 != state_bytes
                 or not kv_seg_states.is_contiguous()):
@@ -260,8 +270,8 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)
         # one state array for the dKV scan, one more when the KV states have to be rebuilt
-        need_dkv = n_seg > 1 or dkv_in is not None or dkv_out is not None
-        need_kv = kv_seg_states is None and (n_seg > 1 or kv_in is not None)
+        need_dkv = not fused and (n_seg > 1 or dkv_in is not None or dkv_out is not None)
+        need_kv = not fused and kv_seg_states is None and (n_seg > 1 or kv_in is not None)
         n_arrays = int(need_dkv) + int(need_kv)
         ws = torch.empty((n_arrays * state_bytes // 4,), dtype=torch.float32, device=dev) if n_arrays else None
         rc = lib.lasp_chunk_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), _ptr(kv_in),

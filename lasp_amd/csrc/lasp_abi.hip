@@ -104,9 +104,27 @@ bool mfma_f32_eligible(int d, int e, int dtype) {
   return dtype == LASP_DTYPE_F32 && d == kMaxFeature && e == kMaxFeature;
 }
 
+// Short chunks given to the library with the default plan run as ONE launch per direction: every
+// workgroup rebuilds the state entering its segment by walking the blocks before it, which saves
+// the pre-pass, the scan, their launches and the workspace.  The walk is serial work on the
+// critical path (about 1.3 us per 64-token block against 4-5 us for a block of the sweep), so the
+// path is only taken while the longest walk stays within 8 blocks, or within the length of one
+// segment's own sweep: measured at b*h = 24 it wins up to n = 512 (49 against 60 us forward +
+// backward) and loses from n = 1024 (73 against 66 us).  An explicit seg_len always selects the
+// pre-pass / scan / sweep kernels.
+constexpr int64_t kFusedMaxTokens = 2048;
+constexpr int kFusedMaxWalk = 8;  // blocks
+bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg_len, int64_t n_seg) {
+  if (seg_len_arg != 0 || !mfma_eligible(d, e, dtype) || n > kFusedMaxTokens) return false;
+  const int per_seg = seg_len / kSegQuantum;  // blocks in one segment's sweep
+  const int64_t longest_walk = (n_seg - 1) * per_seg;
+  return longest_walk <= (per_seg > kFusedMaxWalk ? per_seg : kFusedMaxWalk);
+}
+
 int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
   int rc = check_shape(b, h, n, d, e, dtype);
   if (rc) return rc;
+  const int seg_len_arg = seg_len;
   if (seg_len == 0) seg_len = default_seg_len(b, h, n);
   if (seg_len < 0 || seg_len % kSegQuantum != 0) {
     set_error("seg_len=%d must be a positive multiple of %d (or 0 for the default)", seg_len,
@@ -125,6 +143,7 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   g->e = e;
   g->seg_len = seg_len;
   g->n_seg = (int)n_seg;
+  g->fused = fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg) ? 1 : 0;
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;
@@ -292,6 +311,7 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
   Geom g;
   int rc = make_geom(b, h, n, d, e, dtype, 0, &g);
   if (rc) return rc;
+  if (g.fused) return LASP_PATH_MFMA_FUSED;
   return (mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
 }
 
@@ -325,7 +345,7 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
     set_error("lasp_chunk_fwd: q, k, v, s and o must not be NULL");
     return LASP_E_NULL;
   }
-  if (!seg_states && (g.n_seg > 1 || kv_in || kv_out)) {
+  if (!g.fused && !seg_states && (g.n_seg > 1 || kv_in || kv_out)) {
     set_error("lasp_chunk_fwd: seg_states workspace (%zu bytes) is required for n_seg=%d%s",
               state_bytes_of(g), g.n_seg, (kv_in || kv_out) ? " with KV in/out" : "");
     return LASP_E_WORKSPACE;
@@ -343,7 +363,7 @@ int lasp_chunk_fwd_static(const void *q, const void *k, const void *v, const flo
     set_error("lasp_chunk_fwd_static: q, k, v, s and o must not be NULL");
     return LASP_E_NULL;
   }
-  if (state_bytes_of(g) > (size_t)LASP_STATIC_SCRATCH_BYTES) {
+  if (!g.fused && state_bytes_of(g) > (size_t)LASP_STATIC_SCRATCH_BYTES) {
     set_error("lasp_chunk_fwd_static: the segment states of this call take %zu bytes (b*h*n_seg = %lld states), "
               "the library's scratch holds %zu; pass a larger seg_len or use lasp_chunk_fwd with a workspace",
               state_bytes_of(g), (long long)g.b * g.h * g.n_seg, (size_t)LASP_STATIC_SCRATCH_BYTES);
@@ -369,8 +389,8 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
     return LASP_E_NULL;
   }
   const size_t one = state_bytes_of(g);
-  const bool need_kv = !kv_seg_states && (g.n_seg > 1 || kv_in);
-  const bool need_dkv = g.n_seg > 1 || dkv_in || dkv_out;
+  const bool need_kv = !g.fused && !kv_seg_states && (g.n_seg > 1 || kv_in);
+  const bool need_dkv = !g.fused && (g.n_seg > 1 || dkv_in || dkv_out);
   const size_t need = one * ((need_kv ? 1 : 0) + (need_dkv ? 1 : 0));
   if (need && (!workspace || workspace_bytes < need)) {
     set_error("lasp_chunk_bwd: workspace of %zu bytes required, got %zu", need,

@@ -57,6 +57,7 @@ struct Geom {
   int n_seg;    // ceil(n / seg_len)
   int sd, se;   // rows and columns of one segment state as stored in the workspace: d x e for the
                 // generic kernels, 128 x 128 (zero beyond d, e) for the MFMA kernels
+  int fused;    // the chunk is served by the single-launch kernels, which use no workspace
 };
 
 // Host-side launchers (each returns a hipError_t as int, or a negative LASP_E_*).
@@ -114,7 +115,7 @@ int grant_lds(int max_bytes) {
 
 // Optional per-kernel timing (lasp_profile_begin / lasp_profile_end): while a
 // profile is open every kernel launch is bracketed by two events on its stream.
-enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_BWD3 = 4, KC_COUNT = 5 };
+enum KernelClass { KC_APPLY = 0, KC_STATE = 1, KC_SCAN = 2, KC_GENERIC = 3, KC_BWD3 = 4, KC_FUSED = 5, KC_COUNT = 6 };
 struct ProfEntry;
 struct ProfScope {
   ProfScope(int kernel_class, hipStream_t st);

@@ -59,6 +59,7 @@ constexpr int OFF_ZT = OFF_YT + F * LDT;
 constexpr int OFF_SC = OFF_ZT + F * LDT;
 constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float SKIP_LOG2 = 64.f;  // decay weights below 2^-SKIP_LOG2 are treated as zero (see la_seg_state)
 enum Mode { M_ALIGNED = 0, M_RAGGED = 1, M_NARROW = 2 };
 
 // Element policies: the kernels move 16-bit elements as raw bits and only touch their value
@@ -248,7 +249,8 @@ struct SegWork {
 // `item` enumerates (b*h, segment) pairs
 __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
   SegWork r;
-  r.bh = item / g.n_seg;
+  // the division runs on the vector unit; its (uniform) result goes back to a scalar register
+  r.bh = __builtin_amdgcn_readfirstlane(item / g.n_seg);
   r.seg = item - r.bh * g.n_seg;
   r.tok0 = (int64_t)r.seg * g.seg_len;
   int64_t t1 = r.tok0 + g.seg_len;
@@ -265,11 +267,20 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 // (multiples of 8, at most 128); the upper half of the feature steps and state tiles, and waves
 // whose columns lie in the zero extension, are skipped when they would only see zeros.
 // M_ALIGNED carries none of that bookkeeping; fa and fb are read in M_NARROW only.
-template <class E, bool REV, bool TRANS, int MODE>
+//
+// FUSED: the state entering the segment is not read from a workspace but rebuilt inside the
+// workgroup, by first walking the blocks that precede the segment (follow it, going backwards)
+// and only updating the state: no X tile, no score, no output.  The walk starts from the chunk's
+// incoming state `carry_in` (d x e floats per (b, h), may be NULL), or from zero as many blocks
+// back as the head's decay reaches (weights below 2^-SKIP_LOG2 are dropped).  The workgroup
+// of the segment visited last writes the state it ends with to `carry_out` (non-transposed roles
+// only).  One launch then does a whole chunk; the repeated walks make it a tool for short chunks.
+template <class E, bool REV, bool TRANS, int MODE, bool FUSED = false>
 __device__ __forceinline__ void
 apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
-           const Geom &g, int fa, int fb, int item, char *smem) {
+           const Geom &g, int fa, int fb, int item, char *smem, const float *__restrict__ carry_in = nullptr,
+           float *__restrict__ carry_out = nullptr) {
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -309,9 +320,37 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
   const int qI = w >> 1, qJ = w & 1;  // score quadrant of this wave: queries 32*qI.., keys 32*qJ..
   const bool q_active = REV ? !(qI == 1 && qJ == 0) : !(qI == 0 && qJ == 1);
 
+  // ---- FUSED: how many blocks outside the segment the state is walked over first
+  const int total_blk = (int)((g.n + BLK - 1) / BLK);          // blocks in the chunk
+  const int seg_blk0 = (int)(sw.tok0 / BLK);                    // the segment's first block
+  const int chunk_tail = (int)(g.n - (int64_t)(total_blk - 1) * BLK);
+  int runup = 0;
+  bool take_carry = false;
+  if (FUSED) {
+    const int avail = REV ? total_blk - (seg_blk0 + sw.nblk) : seg_blk0;
+    int reach = avail;
+    if (sl > 0.f) {
+      const float x = SKIP_LOG2 / (sl * (float)BLK);  // blocks over which a weight falls to 2^-SKIP_LOG2
+      if (x < (float)avail) reach = (int)x + 1;
+    }
+    runup = __builtin_amdgcn_readfirstlane(min(reach, avail));
+    take_carry = carry_in != nullptr && runup == avail;
+  }
+
   // ---- state entering the segment, as accumulator tiles: st[T][4g+r] = St[32T+8g+4hh+r][32w+c]
   floatx16 st[4];
-  if (states) {
+  if (FUSED && take_carry) {
+    const float *cp = carry_in + (int64_t)sw.bh * fa * fb;  // fa x fb (TRANS: fb x fa) floats, unpadded
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * T + 8 * (r >> 2) + 4 * hh + (r & 3);
+        const int col = 32 * w + c;
+        const bool inside = !NARROW || (row < fa && col < fb);
+        st[T][r] = inside ? (TRANS ? cp[col * fa + row] : cp[row * fb + col]) : 0.f;
+      }
+  } else if (!FUSED && states) {
     const float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
 #pragma unroll
     for (int T = 0; T < 4; ++T)
@@ -338,8 +377,15 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
   // every address is a workgroup-uniform block pointer (scalar registers) plus a per-thread 32-bit
   // offset and an immediate; rows past a partial block's end and pieces past a narrow row's width
   // read as zeros
+  // Blocks are numbered relative to the segment (FUSED: negative before it, nblk and up after it).
+  // A partial block is the chunk's last one.
+  auto len_of = [&](int blk) __attribute__((always_inline)) {
+    if (!RAGGED) return BLK;
+    if (!FUSED) return blk == sw.nblk - 1 ? sw.tail : BLK;
+    return seg_blk0 + blk == total_blk - 1 ? chunk_tail : BLK;
+  };
   auto issue_loads = [&](int blk) __attribute__((always_inline)) {
-    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    const int len = len_of(blk);
     const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * xu * 8);
     const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * xu * 8);
     const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * zu * 8);
@@ -355,29 +401,105 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       nz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
     }
   };
-  auto fill_lds = [&]() __attribute__((always_inline)) {
+  auto fill_lds = [&](int blk) __attribute__((always_inline)) {
 #pragma unroll
     for (int it = 0; it < 4; ++it)
       *reinterpret_cast<u32x4 *>(smem + OFF_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
 #pragma unroll
     for (int r = 0; r < 4; ++r)
       *reinterpret_cast<u32x4 *>(smem + OFF_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
-    store_transposed<E, true>(smem + OFF_YT, ny, yr, kdec);
+    const int len = len_of(blk);
+    if (FUSED && RAGGED && !REV && len != BLK) {
+      // the chunk's partial last block, going forwards: its tokens sit `len - b` before the chunk end,
+      // which matters here because the state it leaves is the outgoing one
+      float kd[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
+      store_transposed<E, true>(smem + OFF_YT, ny, yr, kd);
+    } else {
+      store_transposed<E, true>(smem + OFF_YT, ny, yr, kdec);
+    }
     store_transposed<E, false>(smem + OFF_ZT, nz, yr, kdec);
   };
 
-  const int first = REV ? sw.nblk - 1 : 0;
   const int step = REV ? -1 : 1;
-  issue_loads(first);
-  fill_lds();
+  int blk = REV ? sw.nblk - 1 : 0;  // the segment's first block in sweep order
+  issue_loads(blk);  // FUSED: stays in flight during the walk below
+
+  // ---- FUSED: state walk outside the segment: St <- l^len St + (scaled Y)^T Z, nothing else.
+  // A pipeline of its own, shaped like la_seg_state's: two register sets in flight, two LDS
+  // buffers (the second one in the X / Y token-major region, idle here), one barrier per block;
+  // loads past the walk's end repeat its last block so that every wait is exact.
+  if (FUSED && runup > 0) {
+    char *const buf_y[2] = {smem + OFF_YT, smem + OFF_XN};
+    char *const buf_z[2] = {smem + OFF_ZT, smem + OFF_XN + F * LDT};
+    static_assert(2 * F * LDT <= OFF_YT - OFF_XN, "the second walk buffer has to fit the token-major tiles");
+    const int w_first = REV ? sw.nblk - 1 + runup : -runup;
+    auto walk_blk = [&](int i) __attribute__((always_inline)) { return w_first + min(i, runup - 1) * step; };
+    auto walk_loads = [&](u32x4 (&py)[4], u32x4 (&pz)[4], int wb) __attribute__((always_inline)) {
+      const int len = len_of(wb);
+      const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)wb * BLK * xu * 8);
+      const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)wb * BLK * zu * 8);
+      const PieceMask all = {true, true};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
+        py[r] = load_row_pieces(yblk, r * xu * 8, y_off, NARROW ? y_ok : all, row_ok);
+        pz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
+      }
+    };
+    auto walk_fill = [&](int b, const u32x4 (&py)[4], const u32x4 (&pz)[4]) __attribute__((always_inline)) {
+      store_transposed<E, true>(buf_y[b], py, yr, kdec);
+      store_transposed<E, false>(buf_z[b], pz, yr, kdec);
+    };
+    auto walk_step = [&](int b, int wb) __attribute__((always_inline)) {
+      const int len = len_of(wb);
+      const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
+#pragma unroll
+      for (int T = 0; T < 4; ++T)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[T][r] *= bd;
+      if (wave_active) {
+        int cc = c;
+        asm volatile("" : "+v"(cc));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const u32x4 zf = lds16(buf_z[b] + tr_off(32 * w + cc, 2 * u + hh));
+#pragma unroll
+          for (int T = 0; T < 4; ++T)
+            if (!NARROW || T < 2 || fa > 64)
+              st[T] = E::mfma(lds16(buf_y[b] + tr_off(32 * T + cc, 2 * u + hh)), zf, st[T]);
+        }
+      }
+    };
+    u32x4 ya[4], za[4], yb[4], zb[4];
+    walk_loads(ya, za, walk_blk(0));
+    walk_loads(yb, zb, walk_blk(1));
+    walk_fill(0, ya, za);
+    walk_loads(ya, za, walk_blk(2));
+    __syncthreads();
+    for (int i = 0; i < runup; i += 2) {
+      walk_step(0, walk_blk(i));
+      walk_fill(1, yb, zb);
+      walk_loads(yb, zb, walk_blk(i + 3));
+      __syncthreads();
+      if (i + 1 >= runup) break;
+      walk_step(1, walk_blk(i + 1));
+      walk_fill(0, ya, za);
+      walk_loads(ya, za, walk_blk(i + 4));
+      __syncthreads();
+    }
+  }
+  fill_lds(blk);
   __syncthreads();
 
-  for (int it = 0, blk = first; it < sw.nblk; ++it, blk += step) {
+  for (int it = 0; it < sw.nblk; ++it, blk += step) {
     const bool more = it + 1 < sw.nblk;
     if (more) issue_loads(blk + step);
-    // A partial block is the chunk's last one.  Going forwards nothing after it uses the state;
-    // going backwards it comes first and the entering state sits `len` (not 64) tokens ahead.
-    const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
+    // A partial block is the chunk's last one.  Going forwards nothing after it uses the state
+    // (but the outgoing state of a FUSED launch); going backwards it comes first and the entering
+    // state sits `len` (not 64) tokens ahead.
+    const int len = len_of(blk);
     float qd[2] = {qdec[0], qdec[1]};
     float bd = blockdec;
     if (RAGGED && REV && len != BLK) {
@@ -385,6 +507,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       qd[1] = decay(sl, (float)max(len - 32 - c, 0));
       bd = decay(sl, (float)len);
     }
+    if (FUSED && RAGGED && !REV && len != BLK) bd = decay(sl, (float)len);
 
     // (1) one sweep over the 8 feature steps feeds two products from the same X fragments:
     //     state term, transposed:  acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
@@ -512,9 +635,25 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
     }
     if (more) {
       __syncthreads();  // C: staged output consumed
-      fill_lds();
+      fill_lds(blk + step);
       __syncthreads();  // D: next block visible
     }
+  }
+
+  // FUSED: the segment visited last by the chunk's sweep leaves the outgoing state
+  if (FUSED && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
+    float *cp = carry_out + (int64_t)sw.bh * fa * fb;
+    // the lane's position is taken afresh from the hardware lane counter, so that nothing but the
+    // state has to stay in registers across the sweep for this epilogue
+    const int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int col = 32 * w + (ln & 31);
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * T + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3);
+        if (!NARROW || (row < fa && col < fb)) cp[row * fb + col] = st[T][r];
+      }
   }
 }
 
@@ -525,6 +664,48 @@ la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const e
          Geom g) {
   extern __shared__ __align__(16) char smem[];
   apply_body<E, REV, TRANS, MODE>(X, Y, Z, S, states, Out, g, g.d, g.e, (int)blockIdx.x, smem);
+}
+
+// A whole short chunk in one launch: every workgroup rebuilds the state entering its segment
+// (see FUSED above), so there is no pre-pass, no scan and no workspace.
+template <class E, int MODE>
+__global__ void __launch_bounds__(NTHR, 2)
+la_fused_fwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+             const float *__restrict__ S, const float *__restrict__ kv_in, float *__restrict__ kv_out,
+             elem16_t *__restrict__ O, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  // Workgroups are dealt to the 8 XCDs round-robin: all segments of one (b, h) go to the same XCD,
+  // whose L2 then serves the repeated walks over that (b, h)'s K and V; later segments, which walk
+  // over more blocks first, are started first.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int bh = (slot / g.n_seg) * 8 + xcd;
+  if (bh >= g.b * g.h) return;
+  const int item = bh * g.n_seg + (g.n_seg - 1 - slot % g.n_seg);
+  apply_body<E, false, false, MODE, true>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
+}
+
+// roles as in la_bwd3 (the dV role leaves dKV_out); all roles and segments of one (b, h) on one XCD
+template <class E, int MODE>
+__global__ void __launch_bounds__(NTHR, 2)
+la_fused_bwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+             const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_in,
+             const float *__restrict__ dkv_in, float *__restrict__ dkv_out, elem16_t *__restrict__ DQ,
+             elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int per_bh = 3 * g.n_seg;
+  const int bh = (slot / per_bh) * 8 + xcd;
+  if (bh >= g.b * g.h) return;
+  const int rem = slot % per_bh;
+  const int role = rem % 3, k = rem / 3;  // k-th longest walk of its role
+  if (role == 0)  // dQ walks forwards: late segments have the longest walk
+    apply_body<E, false, true, MODE, true>(DO, V, K, S, nullptr, DQ, g, g.e, g.d, bh * g.n_seg + g.n_seg - 1 - k, smem,
+                                           kv_in);
+  else if (role == 1)
+    apply_body<E, true, false, MODE, true>(K, Q, DO, S, nullptr, DV, g, g.d, g.e, bh * g.n_seg + k, smem, dkv_in,
+                                           dkv_out);
+  else
+    apply_body<E, true, true, MODE, true>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
@@ -568,7 +749,6 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
 // the Z tile, each keeping STATE_DEPTH blocks in flight in registers (16 registers per block) on
 // top of the two LDS buffers; wave (wc, rh) owns rows [64 rh, 64 rh + 64) x columns
 // [32 wc, 32 wc + 32) of the state as two accumulator tiles.
-constexpr float SKIP_LOG2 = 64.f;
 constexpr int STATE_THREADS = 512;
 constexpr int STATE_DEPTH = 2;  // blocks in flight per thread in registers (even); deeper measured slower:
                                 // the repeated loads at the end of a walk cost more than the depth gains
@@ -762,7 +942,33 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
 }
 
 template <class E, int MODE>
+int launch_fused_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_fused_fwd<E, MODE>>(APPLY_LDS);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * g.n_seg);  // whole groups of 8 (b, h)
+  ProfScope prof(KC_FUSED, st);
+  la_fused_fwd<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, a.s, a.kv_in, a.kv_out,
+                                                         (elem16_t *)a.o, g);
+  return (int)hipGetLastError();
+}
+
+template <class E, int MODE>
+int launch_fused_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_fused_bwd<E, MODE>>(APPLY_LDS);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * 3 * g.n_seg);
+  ProfScope prof(KC_FUSED, st);
+  la_fused_bwd<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
+                                                         a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
+                                                         (elem16_t *)a.dk, (elem16_t *)a.dv, g);
+  return (int)hipGetLastError();
+}
+
+template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  if (g.fused) return launch_fused_fwd<E, MODE>(a, g, st);
   int rc;
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
@@ -774,6 +980,7 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
 
 template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
+  if (g.fused) return launch_fused_bwd<E, MODE>(a, g, st);
   int rc;
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {

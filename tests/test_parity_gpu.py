@@ -33,6 +33,20 @@ def run_abi(inp, s, dev, seg_len=0, cache=False, exact=False):
     return dict(o=o, kv_out=kv_out, dq=dq, dk=dk, dv=dv, dkv_out=dkv_out)
 
 
+def mfma_path(b, h, n, dtype, d=128, e=128):
+    """The path id of an MFMA-eligible shape under the default plan.  Short 16-bit chunks whose segments
+    are few (longest walk over preceding blocks within 8 blocks, or within one segment's own length) run
+    as one launch per direction; an explicit seg_len, as most tests below pass, always selects the
+    pre-pass / scan / sweep kernels."""
+    from lasp_amd import _abi
+
+    if dtype == torch.float32 or n > 2048:
+        return _abi.PATH_MFMA
+    seg_len, n_seg, _ = _abi.plan(b, h, n, d, e, dtype)
+    per_seg = seg_len // 64
+    return _abi.PATH_MFMA_FUSED if (n_seg - 1) * per_seg <= max(8, per_seg) else _abi.PATH_MFMA
+
+
 def test_library_loaded_and_path_selection(gpu_device):
     from lasp_amd import _abi
 
@@ -41,7 +55,10 @@ def test_library_loaded_and_path_selection(gpu_device):
     assert _abi.kernel_path(1, 16, 65536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.float32) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 96, torch.float32) == _abi.PATH_GENERIC
-    assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_MFMA       # 8 segments: too long a walk
+    assert _abi.kernel_path(2, 12, 512, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 segments
+    assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 long segments
+    assert _abi.kernel_path(4, 32, 2049, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC
 
@@ -126,7 +143,7 @@ def test_argument_errors(gpu_device):
 def test_mfma_bf16(gpu_device, b, h, n, seg, state):
     from lasp_amd import _abi
 
-    assert _abi.kernel_path(b, h, n, 128, 128, torch.bfloat16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(b, h, n, 128, 128, torch.bfloat16) == mfma_path(b, h, n, torch.bfloat16)
     inp = make_inputs(b, h, n, 128, 128, torch.bfloat16, seed=n + h, state=state, state_std=1.0)
     s = O.slopes_baseline(h) if h > 1 else torch.tensor([0.05])
     got = run_abi(inp, s, gpu_device, seg_len=seg)
@@ -167,7 +184,7 @@ def test_narrow_bf16_heads_on_mfma(gpu_device, d, e):
     from lasp_amd import _abi
 
     native = d % 8 == 0 and e % 8 == 0
-    assert _abi.kernel_path(2, 3, 512, d, e, torch.bfloat16) == (_abi.PATH_MFMA if native else _abi.PATH_GENERIC)
+    assert _abi.kernel_path(2, 3, 512, d, e, torch.bfloat16) == (_abi.PATH_MFMA_FUSED if native else _abi.PATH_GENERIC)
     inp = make_inputs(2, 3, 512, d, e, torch.bfloat16, seed=d + e, state=True, state_std=1.0)
     assert _abi._pad_to_mfma(inp["q"], inp["v"]) == (not native)
     s = O.slopes_alibi(3)
@@ -177,29 +194,47 @@ def test_narrow_bf16_heads_on_mfma(gpu_device, d, e):
         check(got, oracle(inp, s), 2e-2, what=f"narrow d={d} e={e} cache={cache}")
 
 
-def test_narrow_rows_leave_neighbouring_memory_alone(gpu_device):
+@pytest.mark.parametrize("seg", [0, 64])
+def test_narrow_rows_leave_neighbouring_memory_alone(gpu_device, seg):
     """Outputs narrower than 128 features are written at their own width: a guard band after
-    each output tensor keeps its bits."""
+    each output tensor keeps its bits (seg 0: the single-launch kernels, 64: pre-pass / scan / sweep)."""
     from lasp_amd import _abi
 
     b, h, n, d, e = 1, 2, 200, 64, 32
     inp = make_inputs(b, h, n, d, e, torch.bfloat16, seed=77, state=True, state_std=1.0, device=gpu_device)
     s = O.slopes_alibi(h).to(gpu_device)
-    o, states, sl = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=torch.empty_like(inp["kv"]))
+    o, states, sl = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=torch.empty_like(inp["kv"]),
+                                   seg_len=seg)
     torch.cuda.synchronize()
+    assert (states is None) == (seg == 0)
     # re-run into views of guarded buffers through the raw entry point
     lib = _abi.load()
     guard = 4096
     buf = torch.full((b * h * n * e + guard,), 1.5, dtype=torch.bfloat16, device=gpu_device)
     kvo = torch.full((b * h * d * e + guard,), -2.5, dtype=torch.float32, device=gpu_device)
     rc = lib.lasp_chunk_fwd(inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(),
-                            inp["kv"].data_ptr(), kvo.data_ptr(), buf.data_ptr(), states.data_ptr(),
+                            inp["kv"].data_ptr(), kvo.data_ptr(), buf.data_ptr(),
+                            None if states is None else states.data_ptr(),
                             b, h, n, d, e, _abi.DTYPE_CODE[torch.bfloat16], sl,
                             torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert rc == 0
     assert torch.equal(buf[:b * h * n * e].view(b, h, n, e), o)
     assert (buf[b * h * n * e:] == 1.5).all() and (kvo[b * h * d * e:] == -2.5).all()
+    # the gradients as well
+    dkvo = torch.full((b * h * d * e + guard,), -2.5, dtype=torch.float32, device=gpu_device)
+    outs = [torch.full((b * h * n * w_ + guard,), 1.5, dtype=torch.bfloat16, device=gpu_device) for w_ in (d, d, e)]
+    ws = torch.empty(2 * b * h * 8 * 128 * 128, dtype=torch.float32, device=gpu_device)
+    rc = lib.lasp_chunk_bwd(inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(),
+                            inp["do"].data_ptr(), inp["kv"].data_ptr(), inp["dkv"].data_ptr(), outs[0].data_ptr(),
+                            outs[1].data_ptr(), outs[2].data_ptr(), dkvo.data_ptr(), None, ws.data_ptr(),
+                            ws.numel() * 4, b, h, n, d, e, _abi.DTYPE_CODE[torch.bfloat16], sl,
+                            torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0, lib.lasp_last_error()
+    for t, w_ in zip(outs, (d, d, e)):
+        assert (t[b * h * n * w_:] == 1.5).all() and torch.isfinite(t[:b * h * n * w_].float()).all()
+    assert (dkvo[b * h * d * e:] == -2.5).all()
 
 
 @pytest.mark.parametrize("n,d,e", [(2047, 128, 128), (65, 128, 128), (700, 128, 64), (63, 128, 128), (1, 128, 128)])
@@ -217,7 +252,7 @@ def test_ragged_bf16_length(gpu_device, n, d, e):
 def test_mfma_fp16(gpu_device, b, h, n, seg, state):
     from lasp_amd import _abi
 
-    assert _abi.kernel_path(b, h, n, 128, 128, torch.float16) == _abi.PATH_MFMA
+    assert _abi.kernel_path(b, h, n, 128, 128, torch.float16) == mfma_path(b, h, n, torch.float16)
     inp = make_inputs(b, h, n, 128, 128, torch.float16, seed=n + 7, state=state, state_std=1.0)
     s = O.slopes_baseline(h)
     got = run_abi(inp, s, gpu_device, seg_len=seg)
@@ -264,7 +299,7 @@ def test_mfma_ragged_lengths_in_kernel(gpu_device, dtype, tol, b, h, n, seg):
     """A chunk length that is not a multiple of the block: the last block is masked inside the kernels."""
     from lasp_amd import _abi
 
-    assert _abi.kernel_path(b, h, n, 128, 128, dtype) == _abi.PATH_MFMA
+    assert _abi.kernel_path(b, h, n, 128, 128, dtype) == mfma_path(b, h, n, dtype)
     inp = make_inputs(b, h, n, 128, 128, dtype, seed=n + 3, state=True, state_std=1.0)
     s = torch.tensor([0.3, 0.01, 2.0][:h])
     ref = oracle(inp, s)
@@ -294,3 +329,69 @@ def test_seeded_random_shapes(gpu_device):
         print(what, flush=True)
         got = run_abi(inp, s, gpu_device, seg_len=seg, cache=bool(case & 1))
         check(got, oracle(inp, s), 1e-4 if dtype == torch.float32 else 2e-2, what=what)
+
+
+# ---------------------------------------------------------------- single-launch path for short chunks
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("state", [False, True])
+@pytest.mark.parametrize("b,h,n,d,e", [
+    (2, 12, 512, 128, 128),    # two segments of 256 tokens
+    (4, 32, 2048, 128, 128),   # two segments of 1024 tokens: a walk as long as the sweep
+    (1, 3, 768, 128, 128),     # three segments
+    (1, 2, 64, 128, 128), (1, 1, 192, 128, 128),
+    (2, 3, 700, 128, 128), (1, 4, 513, 128, 128), (1, 2, 333, 128, 128), (1, 2, 1, 128, 128),   # ragged lengths
+    (2, 12, 512, 128, 64), (1, 3, 700, 64, 96), (2, 2, 321, 48, 16),                              # narrow rows
+])
+def test_fused_short_chunks_match_oracle_and_three_kernel_path(gpu_device, b, h, n, d, e, state, dtype):
+    """Default plan, short chunk, few segments: one launch per direction, states rebuilt inside each workgroup.  Checked
+    against the oracle and against the pre-pass / scan / sweep kernels on the same segment length."""
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(b, h, n, d, e, dtype) == _abi.PATH_MFMA_FUSED
+    inp = make_inputs(b, h, n, d, e, dtype, seed=n + d + e, scale=0.5, state=state, state_std=1.0)
+    s = O.slopes_baseline(h) if h > 1 else torch.tensor([0.004])
+    got = run_abi(inp, s, gpu_device)                      # seg_len 0: the single-launch kernels
+    check(got, oracle(inp, s), 2e-2, what=f"fused b={b} h={h} n={n} d={d} e={e} state={state}")
+    planned = _abi.plan(b, h, n, d, e, dtype)[0]
+    other = run_abi(inp, s, gpu_device, seg_len=planned)   # explicit seg_len: the three-kernel path
+    for name in ("o", "dq", "dk", "dv", "kv_out", "dkv_out"):
+        if got[name] is not None:
+            assert O.rel_err(got[name], other[name].float()) <= 2e-2, name
+
+
+def test_fused_special_slopes(gpu_device):
+    # no decay (nothing may be skipped, the walk always reaches the chunk's start and the incoming state),
+    # moderate and very fast decay (the walk is cut to a block or two)
+    inp = make_inputs(1, 3, 768, 128, 128, torch.bfloat16, seed=19, scale=0.3, state=True, state_std=1.0)
+    s = torch.tensor([0.0, 1.0, 30.0])
+    from lasp_amd import _abi
+
+    assert _abi.kernel_path(1, 3, 768, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED
+    got = run_abi(inp, s, gpu_device)
+    assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
+    check(got, oracle(inp, s), 2e-2, what="fused s in {0, 1, 30}")
+
+
+def test_fused_needs_no_workspace_through_the_raw_abi(gpu_device):
+    from lasp_amd import _abi
+
+    lib = _abi.load()
+    dev = gpu_device
+    b, h, n, d = 1, 4, 512, 128
+    assert _abi.kernel_path(b, h, n, d, d, torch.bfloat16) == _abi.PATH_MFMA_FUSED
+    inp = make_inputs(b, h, n, d, d, torch.bfloat16, seed=23, scale=d ** -0.5, state=True, device=dev)
+    s = O.slopes_baseline(h).reshape(-1).to(dev)
+    o = torch.empty_like(inp["v"])
+    kvo, dkvo = torch.empty_like(inp["kv"]), torch.empty_like(inp["dkv"])
+    dq, dk, dv = torch.empty_like(inp["q"]), torch.empty_like(inp["k"]), torch.empty_like(inp["v"])
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    code = _abi.DTYPE_CODE[torch.bfloat16]
+    rc = lib.lasp_chunk_fwd(inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(),
+                            inp["kv"].data_ptr(), kvo.data_ptr(), o.data_ptr(), None, b, h, n, d, d, code, 0, stream)
+    assert rc == 0, lib.lasp_last_error()
+    rc = lib.lasp_chunk_bwd(inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(),
+                            inp["do"].data_ptr(), inp["kv"].data_ptr(), inp["dkv"].data_ptr(), dq.data_ptr(),
+                            dk.data_ptr(), dv.data_ptr(), dkvo.data_ptr(), None, None, 0, b, h, n, d, d, code, 0, stream)
+    assert rc == 0, lib.lasp_last_error()
+    torch.cuda.synchronize()
+    check(dict(o=o, kv_out=kvo, dq=dq, dk=dk, dv=dv, dkv_out=dkvo), oracle(inp, s), 2e-2, what="raw fused calls")
