@@ -149,3 +149,22 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text, f"{f} mentions the oracle"
+
+
+def test_bench_reads_its_traffic_figures_from_the_committed_profile():
+    """bench.py's roofline.traffic comes from profiles/pmc_hbm_bytes_config2.txt, not from constants in the
+    script: the file parses, names the segment plan the library still chooses for the headline shape, and its
+    figures are at least the algorithmic bytes of each kernel."""
+    import sys
+
+    sys.path.insert(0, ROOT)
+    import bench
+    from lasp_amd import _abi
+
+    prof = bench.read_traffic_profile()
+    assert prof is not None, "profiles/pmc_hbm_bytes_config2.txt is missing or has no plan/scale/traffic lines"
+    assert (prof["seg_len"], prof["n_seg"]) == _abi.plan(bench.B, bench.H, bench.N, bench.D, bench.D, torch.bfloat16)[:2]
+    th = bench.B * bench.H * bench.N
+    assert prof["kernels"]["la_bwd3"] >= bench.BYTES_BWD_PER_TH * th
+    assert prof["kernels"]["la_apply"] >= bench.BYTES_FWD_PER_TH * th
+    assert prof["kernels"]["la_bwd3"] < 2 * bench.BYTES_BWD_PER_TH * th

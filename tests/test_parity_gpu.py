@@ -395,3 +395,15 @@ def test_fused_needs_no_workspace_through_the_raw_abi(gpu_device):
     assert rc == 0, lib.lasp_last_error()
     torch.cuda.synchronize()
     check(dict(o=o, kv_out=kvo, dq=dq, dk=dk, dv=dv, dkv_out=dkvo), oracle(inp, s), 2e-2, what="raw fused calls")
+
+
+def test_fp16_large_incoming_state_stays_finite(gpu_device):
+    """fp16 I/O rounds the fp32 state to fp16 before each matrix product: an incoming state three orders of
+    magnitude above the activations is well inside the fp16 range and must come through with the usual bound
+    (the range limit itself, |state| or |q.k| beyond 65504, is part of the contract in include/lasp_hip.h)."""
+    inp = make_inputs(1, 3, 1024, 128, 128, torch.float16, seed=91, scale=128 ** -0.5, state=True, state_std=1e3)
+    s = O.slopes_baseline(3)
+    for seg in (0, 256):
+        got = run_abi(inp, s, gpu_device, seg_len=seg)
+        assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
+        check(got, oracle(inp, s), 2e-2, what=f"fp16 with kv_in of std 1e3, seg={seg}")
