@@ -178,15 +178,17 @@ def chain_step(lasp_amd, op, parts, s, KV, DKV):
     loopback standing in for the neighbouring ranks (one process plays every sequence-parallel rank)."""
     chunks = len(parts)
 
+    grads = [p[3] for p in parts]
+
     def step():
         outs = []
         for c, (q, k, v, _do) in enumerate(parts):
             q.grad = k.grad = v.grad = None
             lasp_amd.set_sequence_parallel_rank(c)
             outs.append(op(q, k, v, s, KV, DKV))
-        for c in reversed(range(chunks)):
-            lasp_amd.set_sequence_parallel_rank(c)
-            outs[c].backward(parts[c][3])
+        # one backward over the whole chain, as a model that sums the chunks' losses would run it: autograd
+        # visits the chunk operators last-created first, which is the order the dKV chain needs
+        torch.autograd.backward(outs, grads)
 
     return step
 
