@@ -110,10 +110,11 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype);
  *           KV_out = l^n KV_in + sum_j l^(n-j) k_j^T v_j              (l = exp(-s_h))
  * kv_in  NULL = zero incoming state.  kv_out NULL = state not wanted.
  * kv_out may alias kv_in (in-place update, as lasp/lasp_fuse.py:126-127).
- * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds the
- * state entering each segment (segment 0: KV_in), which lasp_chunk_bwd accepts
- * as `kv_seg_states` to skip recomputing it.  It may be NULL only when
- * n_seg == 1 and kv_in == NULL and kv_out == NULL.
+ * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds per-segment states (opaque:
+ * the state entering each segment, or with few segments each segment's own contribution), which
+ * lasp_chunk_bwd accepts as `kv_seg_states` -- for the same inputs, seg_len and kv_in -- to skip
+ * recomputing them.  It may be NULL when n_seg == 1 and kv_in == NULL and kv_out == NULL, and on
+ * LASP_PATH_MFMA_FUSED.
  */
 int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s,
                    const float *kv_in, float *kv_out, void *o, float *seg_states,

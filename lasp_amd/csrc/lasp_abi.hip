@@ -106,19 +106,23 @@ bool mfma_f32_eligible(int d, int e, int dtype) {
 
 // Short chunks given to the library with the default plan run as ONE launch per direction: every
 // workgroup rebuilds the state entering its segment by walking the blocks before it, which saves
-// the pre-pass, the scan, their launches and the workspace.  The walk is serial work on the
-// critical path (about 1.3 us per 64-token block against 4-5 us for a block of the sweep), so the
-// path is only taken while the longest walk stays within 8 blocks, or within the length of one
-// segment's own sweep: measured at b*h = 24 it wins up to n = 512 (49 against 60 us forward +
-// backward) and loses from n = 1024 (73 against 66 us).  An explicit seg_len always selects the
-// pre-pass / scan / sweep kernels.
+// the pre-pass, its launch and the workspace.  The walk is serial work on the critical path (about
+// 1.3 us per 64-token block against 4-5 us for a block of the sweep), so the path is only taken
+// while the longest walk stays within 8 blocks: measured at b*h = 24 it wins up to n = 512 (49
+// against 53 us forward + backward) and loses beyond.  An explicit seg_len always selects the
+// pre-pass / sweep kernels.
 constexpr int64_t kFusedMaxTokens = 2048;
 constexpr int kFusedMaxWalk = 8;  // blocks
+// With few segments the 16-bit sweeps of full-width heads gather the segments' own states themselves
+// (each workgroup re-runs the scan's recurrence over at most kCombineMaxSeg - 1 states of 64 KiB)
+// and the scan launch is dropped; with one segment the pre-pass goes too.  Measured at b*h = 24,
+// n = 2048: 4 segments 84 against 88 us forward + backward, 8 segments 137 against 100 us (the
+// gathers grow with the square of the segment count), hence the limit.
+constexpr int64_t kCombineMaxSeg = 4;
 bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg_len, int64_t n_seg) {
   if (seg_len_arg != 0 || !mfma_eligible(d, e, dtype) || n > kFusedMaxTokens) return false;
   const int per_seg = seg_len / kSegQuantum;  // blocks in one segment's sweep
-  const int64_t longest_walk = (n_seg - 1) * per_seg;
-  return longest_walk <= (per_seg > kFusedMaxWalk ? per_seg : kFusedMaxWalk);
+  return (n_seg - 1) * per_seg <= kFusedMaxWalk;
 }
 
 int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
@@ -144,6 +148,8 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   g->seg_len = seg_len;
   g->n_seg = (int)n_seg;
   g->fused = fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg) ? 1 : 0;
+  g->combine = (!g->fused && mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature &&
+                n_seg <= kCombineMaxSeg) ? 1 : 0;
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;
@@ -345,7 +351,7 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s, 
     set_error("lasp_chunk_fwd: q, k, v, s and o must not be NULL");
     return LASP_E_NULL;
   }
-  if (!g.fused && !seg_states && (g.n_seg > 1 || kv_in || kv_out)) {
+  if (!g.fused && !seg_states && (g.n_seg > 1 || (!g.combine && (kv_in || kv_out)))) {
     set_error("lasp_chunk_fwd: seg_states workspace (%zu bytes) is required for n_seg=%d%s",
               state_bytes_of(g), g.n_seg, (kv_in || kv_out) ? " with KV in/out" : "");
     return LASP_E_WORKSPACE;
@@ -389,8 +395,8 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
     return LASP_E_NULL;
   }
   const size_t one = state_bytes_of(g);
-  const bool need_kv = !g.fused && !kv_seg_states && (g.n_seg > 1 || kv_in);
-  const bool need_dkv = !g.fused && (g.n_seg > 1 || dkv_in || dkv_out);
+  const bool need_kv = !g.fused && !kv_seg_states && (g.n_seg > 1 || (!g.combine && kv_in));
+  const bool need_dkv = !g.fused && (g.n_seg > 1 || (!g.combine && (dkv_in || dkv_out)));
   const size_t need = one * ((need_kv ? 1 : 0) + (need_dkv ? 1 : 0));
   if (need && (!workspace || workspace_bytes < need)) {
     set_error("lasp_chunk_bwd: workspace of %zu bytes required, got %zu", need,

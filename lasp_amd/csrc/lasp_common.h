@@ -58,6 +58,7 @@ struct Geom {
   int sd, se;   // rows and columns of one segment state as stored in the workspace: d x e for the
                 // generic kernels, 128 x 128 (zero beyond d, e) for the MFMA kernels
   int fused;    // the chunk is served by the single-launch kernels, which use no workspace
+  int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
 };
 
 // Host-side launchers (each returns a hipError_t as int, or a negative LASP_E_*).

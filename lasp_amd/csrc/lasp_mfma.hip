@@ -61,6 +61,8 @@ constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per C
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float SKIP_LOG2 = 64.f;  // decay weights below 2^-SKIP_LOG2 are treated as zero (see la_seg_state)
 enum Mode { M_ALIGNED = 0, M_RAGGED = 1, M_NARROW = 2 };
+// where a sweep takes the state entering its segment from (see apply_body)
+enum Source { SRC_SCANNED = 0, SRC_WALK = 1, SRC_COMBINE = 2 };
 
 // Element policies: the kernels move 16-bit elements as raw bits and only touch their value
 // in three places -- widening one element, rounding two floats into a packed pair, and the
@@ -104,6 +106,12 @@ __device__ __forceinline__ gmem_ptr uniform_ptr(const char *p) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return (gmem_ptr)(((uint64_t)hi << 32) | lo);
+}
+
+// The lane's index within its wave, read from the hardware lane counter: two instructions, and no
+// register has to carry it from the top of the kernel to the place that needs it.
+__device__ __forceinline__ int fresh_lane() {
+  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
 
 __device__ __forceinline__ u32x4 lds16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
@@ -268,20 +276,28 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 // whose columns lie in the zero extension, are skipped when they would only see zeros.
 // M_ALIGNED carries none of that bookkeeping; fa and fb are read in M_NARROW only.
 //
-// FUSED: the state entering the segment is not read from a workspace but rebuilt inside the
-// workgroup, by first walking the blocks that precede the segment (follow it, going backwards)
-// and only updating the state: no X tile, no score, no output.  The walk starts from the chunk's
-// incoming state `carry_in` (d x e floats per (b, h), may be NULL), or from zero as many blocks
-// back as the head's decay reaches (weights below 2^-SKIP_LOG2 are dropped).  The workgroup
-// of the segment visited last writes the state it ends with to `carry_out` (non-transposed roles
-// only).  One launch then does a whole chunk; the repeated walks make it a tool for short chunks.
-template <class E, bool REV, bool TRANS, int MODE, bool FUSED = false>
+// SRC says where the state entering the segment comes from.
+// SRC_SCANNED: `states` holds it, left there by the decayed scan over the segments' own states.
+// SRC_COMBINE: `states` holds the segments' OWN states as the pre-pass wrote them, and the
+//   workgroup runs the scan's recurrence itself over the segments before (after) its own,
+//   starting from the chunk's incoming state `carry_in` (d x e floats per (b, h), may be NULL):
+//   St <- l^len_j St + own_j.  With few segments that is cheaper than a scan launch.
+// SRC_WALK: no workspace at all: the state is rebuilt by first walking the blocks that precede the
+//   segment (follow it, going backwards) and only updating the state: no X tile, no score, no
+//   output.  The walk starts from `carry_in`, or from zero as many blocks back as the head's decay
+//   reaches (weights below 2^-SKIP_LOG2 are dropped).  One launch then does a whole chunk; the
+//   repeated walks make it a tool for short chunks.
+// In the last two the workgroup of the segment visited last writes the state it ends with to
+// `carry_out` (non-transposed roles only).
+template <class E, bool REV, bool TRANS, int MODE, int SRC = SRC_SCANNED>
 __device__ __forceinline__ void
 apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
            const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
            const Geom &g, int fa, int fb, int item, char *smem, const float *__restrict__ carry_in = nullptr,
            float *__restrict__ carry_out = nullptr) {
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
+  constexpr bool FUSED = SRC == SRC_WALK;          // the state walk and its block numbering
+  constexpr bool LEAVES_STATE = SRC != SRC_SCANNED;  // the sweep's final state is the chunk's outgoing one
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
@@ -339,7 +355,8 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 
   // ---- state entering the segment, as accumulator tiles: st[T][4g+r] = St[32T+8g+4hh+r][32w+c]
   floatx16 st[4];
-  if (FUSED && take_carry) {
+  if (SRC == SRC_COMBINE) take_carry = carry_in != nullptr;
+  if (SRC != SRC_SCANNED && take_carry) {
     const float *cp = carry_in + (int64_t)sw.bh * fa * fb;  // fa x fb (TRANS: fb x fa) floats, unpadded
 #pragma unroll
     for (int T = 0; T < 4; ++T)
@@ -350,7 +367,45 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
         const bool inside = !NARROW || (row < fa && col < fb);
         st[T][r] = inside ? (TRANS ? cp[col * fa + row] : cp[row * fb + col]) : 0.f;
       }
-  } else if (!FUSED && states) {
+  } else if (SRC != SRC_SCANNED) {
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
+  }
+  if (SRC == SRC_COMBINE) {
+    // the scan's recurrence over the segments before (after) this one, in sweep order; a segment's
+    // own state is weighted relative to that segment's far end, so the running state is first
+    // carried across the segment's length (only the chunk's last segment can be shorter)
+    if (states != nullptr) {
+      const float *base = states + (int64_t)sw.bh * g.n_seg * (F * F);
+      const float full = decay(sl, (float)g.seg_len);
+      const float last = decay(sl, (float)(g.n - (int64_t)(g.n_seg - 1) * g.seg_len));
+      const int n_before = REV ? g.n_seg - 1 - sw.seg : sw.seg;
+      // addresses: a scalar pointer per 8-row band (SALU arithmetic) + one per-lane offset + an
+      // immediate, instead of 64 vector address pairs
+      typedef const __attribute__((address_space(1))) float *gmem_f32;
+      const uint32_t lane_off =
+          (uint32_t)(TRANS ? ((32 * w + c) * F + 4 * hh) : (4 * hh * F + 32 * w + c)) * (uint32_t)sizeof(float);
+      for (int i = 0; i < n_before; ++i) {
+        const int j = REV ? g.n_seg - 1 - i : i;
+        const float f = j == g.n_seg - 1 ? last : full;
+        const float *sp = base + (int64_t)j * (F * F);
+#pragma unroll
+        for (int T = 0; T < 4; ++T)
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            const int band = 32 * T + 8 * gq;  // rows band .. band + 7 of the state (this lane: + 4 hh + r)
+            const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(sp + (TRANS ? band : band * F)));
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float own = *reinterpret_cast<gmem_f32>(bp + lane_off + (TRANS ? r : r * F) * sizeof(float));
+              st[T][4 * gq + r] = fmaf(f, st[T][4 * gq + r], own);
+            }
+          }
+      }
+    }
+  } else if (SRC == SRC_SCANNED && states) {
     const float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
 #pragma unroll
     for (int T = 0; T < 4; ++T)
@@ -360,7 +415,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
         const int col = 32 * w + c;
         st[T][r] = TRANS ? sp[col * F + row] : sp[row * F + col];
       }
-  } else {
+  } else if (SRC == SRC_SCANNED) {
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
@@ -409,7 +464,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
     for (int r = 0; r < 4; ++r)
       *reinterpret_cast<u32x4 *>(smem + OFF_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
     const int len = len_of(blk);
-    if (FUSED && RAGGED && !REV && len != BLK) {
+    if (LEAVES_STATE && RAGGED && !REV && len != BLK) {
       // the chunk's partial last block, going forwards: its tokens sit `len - b` before the chunk end,
       // which matters here because the state it leaves is the outgoing one
       float kd[4];
@@ -460,7 +515,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[T][r] *= bd;
       if (wave_active) {
-        int cc = c;
+        int cc = fresh_lane() & 31;
         asm volatile("" : "+v"(cc));
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -507,7 +562,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       qd[1] = decay(sl, (float)max(len - 32 - c, 0));
       bd = decay(sl, (float)len);
     }
-    if (FUSED && RAGGED && !REV && len != BLK) bd = decay(sl, (float)len);
+    if (LEAVES_STATE && RAGGED && !REV && len != BLK) bd = decay(sl, (float)len);
 
     // (1) one sweep over the 8 feature steps feeds two products from the same X fragments:
     //     state term, transposed:  acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
@@ -585,7 +640,7 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       // The swizzled addresses of the feature-major tiles are recomputed for every block (a few
       // integer operations each) rather than held in some twenty registers for the whole sweep:
       // the opaque copy of the lane's column keeps the compiler from hoisting them.
-      int cc = c;
+      int cc = fresh_lane() & 31;
       asm volatile("" : "+v"(cc));
       u32x4 zf[4];
 #pragma unroll
@@ -640,12 +695,12 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
     }
   }
 
-  // FUSED: the segment visited last by the chunk's sweep leaves the outgoing state
-  if (FUSED && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
+  // the segment visited last by the chunk's sweep leaves the outgoing state
+  if (LEAVES_STATE && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
     float *cp = carry_out + (int64_t)sw.bh * fa * fb;
     // the lane's position is taken afresh from the hardware lane counter, so that nothing but the
     // state has to stay in registers across the sweep for this epilogue
-    const int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int ln = fresh_lane();
     const int col = 32 * w + (ln & 31);
 #pragma unroll
     for (int T = 0; T < 4; ++T)
@@ -657,13 +712,15 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
   }
 }
 
-template <class E, bool REV, bool TRANS, int MODE>
+template <class E, bool REV, bool TRANS, int MODE, int SRC>
 __global__ void __launch_bounds__(NTHR, 2)
 la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
-         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
-         Geom g) {
+         const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
+         float *__restrict__ carry_out, elem16_t *__restrict__ Out, Geom g) {
   extern __shared__ __align__(16) char smem[];
-  apply_body<E, REV, TRANS, MODE>(X, Y, Z, S, states, Out, g, g.d, g.e, (int)blockIdx.x, smem);
+  // SRC_COMBINE: later segments have more states to gather first, so they are started first
+  const int item = SRC == SRC_COMBINE ? g.b * g.h * g.n_seg - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  apply_body<E, REV, TRANS, MODE, SRC>(X, Y, Z, S, states, Out, g, g.d, g.e, item, smem, carry_in, carry_out);
 }
 
 // A whole short chunk in one launch: every workgroup rebuilds the state entering its segment
@@ -681,7 +738,7 @@ la_fused_fwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, con
   const int bh = (slot / g.n_seg) * 8 + xcd;
   if (bh >= g.b * g.h) return;
   const int item = bh * g.n_seg + (g.n_seg - 1 - slot % g.n_seg);
-  apply_body<E, false, false, MODE, true>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
+  apply_body<E, false, false, MODE, SRC_WALK>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
 }
 
 // roles as in la_bwd3 (the dV role leaves dKV_out); all roles and segments of one (b, h) on one XCD
@@ -699,24 +756,25 @@ la_fused_bwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, con
   const int rem = slot % per_bh;
   const int role = rem % 3, k = rem / 3;  // k-th longest walk of its role
   if (role == 0)  // dQ walks forwards: late segments have the longest walk
-    apply_body<E, false, true, MODE, true>(DO, V, K, S, nullptr, DQ, g, g.e, g.d, bh * g.n_seg + g.n_seg - 1 - k, smem,
+    apply_body<E, false, true, MODE, SRC_WALK>(DO, V, K, S, nullptr, DQ, g, g.e, g.d, bh * g.n_seg + g.n_seg - 1 - k, smem,
                                            kv_in);
   else if (role == 1)
-    apply_body<E, true, false, MODE, true>(K, Q, DO, S, nullptr, DV, g, g.d, g.e, bh * g.n_seg + k, smem, dkv_in,
+    apply_body<E, true, false, MODE, SRC_WALK>(K, Q, DO, S, nullptr, DV, g, g.d, g.e, bh * g.n_seg + k, smem, dkv_in,
                                            dkv_out);
   else
-    apply_body<E, true, true, MODE, true>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
+    apply_body<E, true, true, MODE, SRC_WALK>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
 }
 
 // The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
 // work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
 // the triple is spread over block indices 8 apart so that all three land on the same
 // XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
-template <class E, int MODE>
+template <class E, int MODE, int SRC>
 __global__ void __launch_bounds__(NTHR, 2)
 la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
         const elem16_t *__restrict__ DO, const float *__restrict__ S,
         const float *__restrict__ kv_states, const float *__restrict__ dkv_states,
+        const float *__restrict__ kv_in, const float *__restrict__ dkv_in, float *__restrict__ dkv_out,
         elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
   extern __shared__ __align__(16) char smem[];
   const int n_items = g.b * g.h * g.n_seg;
@@ -725,11 +783,11 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    apply_body<E, false, true, MODE>(DO, V, K, S, kv_states, DQ, g, g.e, g.d, item, smem);
+    apply_body<E, false, true, MODE, SRC>(DO, V, K, S, kv_states, DQ, g, g.e, g.d, item, smem, kv_in);
   else if (role == 1)
-    apply_body<E, true, false, MODE>(K, Q, DO, S, dkv_states, DV, g, g.d, g.e, item, smem);
+    apply_body<E, true, false, MODE, SRC>(K, Q, DO, S, dkv_states, DV, g, g.d, g.e, item, smem, dkv_in, dkv_out);
   else
-    apply_body<E, true, true, MODE>(V, DO, Q, S, dkv_states, DK, g, g.e, g.d, item, smem);
+    apply_body<E, true, true, MODE, SRC>(V, DO, Q, S, dkv_states, DK, g, g.e, g.d, item, smem, dkv_in);
 }
 
 // ------------------------------------------------------------------------------
@@ -900,31 +958,31 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   }
 }
 
-template <class E, bool REV, bool TRANS, int MODE>
+template <class E, bool REV, bool TRANS, int MODE, int SRC>
 int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
-                 void *out, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_apply<E, REV, TRANS, MODE>>(APPLY_LDS);
+                 const float *carry_in, float *carry_out, void *out, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_apply<E, REV, TRANS, MODE, SRC>>(APPLY_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply<E, REV, TRANS, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
-                                                                 (const elem16_t *)z, s, states,
-                                                                 (elem16_t *)out, g);
+  la_apply<E, REV, TRANS, MODE, SRC><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
+                                                                      (const elem16_t *)z, s, states, carry_in,
+                                                                      carry_out, (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
-template <class E, int MODE>
+template <class E, int MODE, int SRC>
 int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                 hipStream_t st) {
-  int rc = grant_lds<la_bwd3<E, MODE>>(APPLY_LDS);
+  int rc = grant_lds<la_bwd3<E, MODE, SRC>>(APPLY_LDS);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
-                                                    (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
-                                                    kv_states, dkv_states, (elem16_t *)a.dq,
-                                                    (elem16_t *)a.dk, (elem16_t *)a.dv, g);
+  la_bwd3<E, MODE, SRC><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
+                                                         kv_states, dkv_states, a.kv_in, a.dkv_in, a.dkv_out,
+                                                         (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
@@ -966,22 +1024,53 @@ int launch_fused_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// skip_seg: the segment whose own state nothing reads (-1: none)
+template <class E, bool REV, int MODE>
+int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
+                          hipStream_t st) {
+  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_STATE, st);
+  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
+                                                               skip_seg);
+  return (int)hipGetLastError();
+}
+
 template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   if (g.fused) return launch_fused_fwd<E, MODE>(a, g, st);
   int rc;
+  if constexpr (MODE != M_NARROW) if (g.combine) {  // (narrow rows keep the scan: no registers to spare there)
+    // few segments: the pre-pass leaves every segment's own state (the last one's is never read), each
+    // sweep workgroup gathers the ones before it, and the last segment's sweep ends with KV_out
+    if (g.n_seg > 1 &&
+        (rc = launch_state_skipping<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, g.n_seg - 1, st)))
+      return rc;
+    return launch_apply<E, false, false, MODE, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
+                                                            a.kv_in, a.kv_out, a.o, g, st);
+  }
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   if (need_states) {
     if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
-  return launch_apply<E, false, false, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.o, g, st);
+  return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
+                                                          nullptr, nullptr, a.o, g, st);
 }
 
 template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
   if (g.fused) return launch_fused_bwd<E, MODE>(a, g, st);
   int rc;
+  if constexpr (MODE != M_NARROW) if (g.combine) {
+    const float *kv_states = a.kv_seg_states;
+    if (!kv_states && g.n_seg > 1) {
+      if ((rc = launch_state_skipping<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, g, g.n_seg - 1, st))) return rc;
+      kv_states = a.ws_kv;
+    }
+    if (g.n_seg > 1 && (rc = launch_state_skipping<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, 0, st))) return rc;
+    return launch_bwd3<E, MODE, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g,
+                                             st);
+  }
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
     if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
@@ -994,7 +1083,7 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  return launch_bwd3<E, MODE>(a, kv_states, dkv_states, g, st);
+  return launch_bwd3<E, MODE, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
 }
 
 
