@@ -355,24 +355,41 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
 
   // ---- state entering the segment, as accumulator tiles: st[T][4g+r] = St[32T+8g+4hh+r][32w+c]
   floatx16 st[4];
-  if (SRC == SRC_COMBINE) take_carry = carry_in != nullptr;
-  if (SRC != SRC_SCANNED && take_carry) {
-    const float *cp = carry_in + (int64_t)sw.bh * fa * fb;  // fa x fb (TRANS: fb x fa) floats, unpadded
+#pragma unroll
+  for (int T = 0; T < 4; ++T)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
+
+  // st <- f * st + M, M being the 128 x 128 tile whose element (row, col) is src[row * ld + col], or for a
+  // transposed role src[col * ld + row]; `bounded`: src holds only fa x fb (transposed: fb x fa) elements,
+  // the rest of the tile is zero.  Addresses: a scalar pointer per 8-row band (SALU arithmetic) + one
+  // per-lane offset + an immediate.  (The transposed role's loads are scattered, one 128-byte line per lane;
+  // fetching the matrix coalesced into LDS and reading it back transposed was measured and is no faster:
+  // the loads happen once per workgroup and hide behind the other workgroups' streaming.)
+  auto add_state = [&](const float *src, int ld, float f, bool bounded) __attribute__((always_inline)) {
+    typedef const __attribute__((address_space(1))) float *gmem_f32;
+    const uint32_t lane_off =
+        (uint32_t)(TRANS ? (32 * w + c) * ld + 4 * hh : 4 * hh * ld + 32 * w + c) * (uint32_t)sizeof(float);
+    const bool col_ok = !bounded || 32 * w + c < fb;
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = 32 * T + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const int col = 32 * w + c;
-        const bool inside = !NARROW || (row < fa && col < fb);
-        st[T][r] = inside ? (TRANS ? cp[col * fa + row] : cp[row * fb + col]) : 0.f;
+      for (int gq = 0; gq < 4; ++gq) {
+        const int band = 32 * T + 8 * gq;  // rows band .. band + 7 of the state (this lane: + 4 hh + r)
+        const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : (int64_t)band * ld)));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const bool ok = col_ok && (!bounded || band + 4 * hh + r < fa);
+          const float own =
+              ok ? *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * ld) * sizeof(float)) : 0.f;
+          st[T][4 * gq + r] = fmaf(f, st[T][4 * gq + r], own);
+        }
       }
-  } else if (SRC != SRC_SCANNED) {
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
-  }
+  };
+
+  if (SRC == SRC_COMBINE) take_carry = carry_in != nullptr;
+  if (SRC != SRC_SCANNED && take_carry)
+    add_state(carry_in + (int64_t)sw.bh * fa * fb, TRANS ? fa : fb, 0.f, NARROW);  // fa x fb floats, unpadded
   if (SRC == SRC_COMBINE) {
     // the scan's recurrence over the segments before (after) this one, in sweep order; a segment's
     // own state is weighted relative to that segment's far end, so the running state is first
@@ -382,44 +399,13 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       const float full = decay(sl, (float)g.seg_len);
       const float last = decay(sl, (float)(g.n - (int64_t)(g.n_seg - 1) * g.seg_len));
       const int n_before = REV ? g.n_seg - 1 - sw.seg : sw.seg;
-      // addresses: a scalar pointer per 8-row band (SALU arithmetic) + one per-lane offset + an
-      // immediate, instead of 64 vector address pairs
-      typedef const __attribute__((address_space(1))) float *gmem_f32;
-      const uint32_t lane_off =
-          (uint32_t)(TRANS ? ((32 * w + c) * F + 4 * hh) : (4 * hh * F + 32 * w + c)) * (uint32_t)sizeof(float);
       for (int i = 0; i < n_before; ++i) {
         const int j = REV ? g.n_seg - 1 - i : i;
-        const float f = j == g.n_seg - 1 ? last : full;
-        const float *sp = base + (int64_t)j * (F * F);
-#pragma unroll
-        for (int T = 0; T < 4; ++T)
-#pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            const int band = 32 * T + 8 * gq;  // rows band .. band + 7 of the state (this lane: + 4 hh + r)
-            const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(sp + (TRANS ? band : band * F)));
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float own = *reinterpret_cast<gmem_f32>(bp + lane_off + (TRANS ? r : r * F) * sizeof(float));
-              st[T][4 * gq + r] = fmaf(f, st[T][4 * gq + r], own);
-            }
-          }
+        add_state(base + (int64_t)j * (F * F), F, j == g.n_seg - 1 ? last : full, false);
       }
     }
   } else if (SRC == SRC_SCANNED && states) {
-    const float *sp = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = 32 * T + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const int col = 32 * w + c;
-        st[T][r] = TRANS ? sp[col * F + row] : sp[row * F + col];
-      }
-  } else if (SRC == SRC_SCANNED) {
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
+    add_state(states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F), F, 0.f, false);
   }
 
   // ---- block loader: registers <- global, LDS <- registers
