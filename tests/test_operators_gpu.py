@@ -172,6 +172,65 @@ def test_graph_capture_replays_match_eager(gpu_device):
     assert O.rel_err(torch.cat(captured[:chunks], 2), ref["o"]) <= 2e-2
 
 
+@pytest.mark.filterwarnings("ignore:The AccumulateGrad node's stream does not match")
+@pytest.mark.parametrize("op_name", ["lasp_fuse", "lasp_fuse_parallel"])
+def test_operator_chain_in_a_graph(gpu_device, op_name):
+    """The public chunk operators with autograd and the loopback state passing, recorded as one HIP graph
+    (4 chunks forward, one backward over all of them): the gradients after each replay equal the eager ones."""
+    import lasp_amd
+
+    dev = gpu_device
+    b, h, n, d, chunks = 2, 4, 4096, 128, 4
+    inp = make_inputs(b, h, n, d, d, torch.bfloat16, seed=43, state=False)
+    s = O.slopes_baseline(h).to(dev)
+    step = n // chunks
+    leaves = [[inp[x][:, :, c * step:(c + 1) * step].to(dev).requires_grad_(True) for x in ("q", "k", "v")] for c in range(chunks)]
+    dos = [inp["do"][:, :, c * step:(c + 1) * step].to(dev) for c in range(chunks)]
+    KV = torch.empty(b, h, d, d, device=dev)
+    DKV = torch.empty_like(KV)
+    op = getattr(lasp_amd, op_name)
+    lasp_amd.destroy_parallel_groups()
+    lasp_amd.initialize_lasp(1, chunks)
+
+    def run():
+        outs = []
+        for c, (q, k, v) in enumerate(leaves):
+            q.grad = k.grad = v.grad = None
+            lasp_amd.set_sequence_parallel_rank(c)
+            outs.append(op(q, k, v, s, KV, DKV))
+        torch.autograd.backward(outs, dos)
+        return outs
+
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            outs = run()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        eager = [o.detach().clone() for o in outs] + [t.grad.clone() for l in leaves for t in l]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = run()
+        torch.cuda.synchronize()
+        held = [o.detach() for o in outs] + [t.grad for l in leaves for t in l]
+        for _ in range(3):
+            for t in held:
+                t.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for a, e in zip(held, eager):
+                assert torch.equal(a, e)
+            _single_pass({k_: inp[k_][:, :, :512] for k_ in ("q", "k", "v", "do")}, s, dev)  # eager work between replays
+        assert lasp_amd.loopback_pending() == []
+    finally:
+        lasp_amd.destroy_parallel_groups()
+    ref = O.ref_chunked(inp["q"], inp["k"], inp["v"], s.cpu(), inp["do"], dtype=torch.float64)
+    assert O.rel_err(torch.cat(eager[:chunks], 2).cpu(), ref["o"]) <= 2e-2
+    assert O.rel_err(torch.cat(eager[chunks::3], 2).cpu(), ref["dq"]) <= 2e-2
+
+
 @pytest.mark.parametrize("dtype,e", [(torch.bfloat16, 128), (torch.float32, 128), (torch.bfloat16, 64)])
 def test_launch_shims_against_oracle(gpu_device, dtype, e):
     """lasp_fuse.lasp_forward/lasp_backward (states in place) and the lasp_fuse_parallel pair
