@@ -308,6 +308,21 @@ def other_configs(dev):
     r = with_bytes(rates(ms, b, h, n), b, h, n, 2)
     r["chunks"] = chunks
     out["config4a_1m_tokens_chain_lasp_fuse"] = r
+
+    # configuration 4b: the same chain without decay (s = 0), q and k passed through elu(x) + 1
+    with torch.no_grad():
+        for q, k, _v, _do in parts:
+            for t in (q, k):
+                t.copy_(torch.nn.functional.elu(t.float() * D ** 0.5) + 1)
+    s0 = torch.zeros(h, 1, 1, device=dev)
+    lasp_amd.initialize_lasp(1, chunks)
+    try:
+        ms = gpu_time(chain_step(lasp_amd, lasp_amd.lasp_fuse, parts, s0, KV, DKV), 3, warm=1)
+    finally:
+        lasp_amd.destroy_parallel_groups()
+    r = with_bytes(rates(ms, b, h, n), b, h, n, 2)
+    r["chunks"] = chunks
+    out["config4b_1m_tokens_no_decay_chain_lasp_fuse"] = r
     del parts
     torch.cuda.empty_cache()
     return out
