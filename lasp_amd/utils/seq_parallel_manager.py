@@ -225,7 +225,26 @@ def state_send(tensor: torch.Tensor, dst: int, group, src: Optional[int] = None,
         t = tensor.detach()
         group.mailbox.setdefault((me, dst, tag), deque()).append(t if give else t.clone())
         return
+    if _stage_through_host(tensor, group):
+        dist.send(tensor.detach().cpu(), dst=dst, group=group)  # .cpu() waits for the producing kernels
+        return
     dist.send(tensor, dst=dst, group=group)
+
+
+def _stage_through_host(tensor: torch.Tensor, group) -> bool:
+    """Device tensors only go to backends that move device memory themselves (nccl, i.e. RCCL).
+    Over gloo a state is copied to host memory first and back after: gloo's own handling of device
+    tensors can stall when several ranks share one GPU."""
+    return tensor.is_cuda and dist.get_backend(group) == "gloo"
+
+
+def _recv_into(tensor: torch.Tensor, src: int, group) -> None:
+    if _stage_through_host(tensor, group):
+        host = torch.empty(tensor.shape, dtype=tensor.dtype)
+        dist.recv(host, src=src, group=group)
+        tensor.copy_(host)
+        return
+    dist.recv(tensor, src=src, group=group)
 
 
 def _loopback_pop(group: LoopbackGroup, src: int, me: int, tag: int) -> torch.Tensor:
@@ -248,7 +267,7 @@ def state_recv(tensor: torch.Tensor, src: int, group, dst: Optional[int] = None,
         me = get_sequence_parallel_rank() if dst is None else dst
         tensor.copy_(_loopback_pop(group, src, me, tag))
         return
-    dist.recv(tensor, src=src, group=group)
+    _recv_into(tensor, src, group)
 
 
 def state_take(like: torch.Tensor, src: int, group, dst: Optional[int] = None, tag: int = 0) -> torch.Tensor:
@@ -263,7 +282,7 @@ def state_take(like: torch.Tensor, src: int, group, dst: Optional[int] = None, t
         me = get_sequence_parallel_rank() if dst is None else dst
         return _loopback_pop(group, src, me, tag)
     t = torch.empty_like(like)
-    dist.recv(t, src=src, group=group)
+    _recv_into(t, src, group)
     return t
 
 

@@ -125,8 +125,7 @@ def _worker(rank, world, port, dp, sp, ret):
                 spm.state_send(t, info["next"], grp)
                 spm.state_recv(t, info["next"], grp)
             else:
-                got = torch.empty(2, 2)
-                spm.state_recv(got, info["prev"], grp)
+                got = spm.state_take(torch.empty(2, 2), info["prev"], grp)  # a fresh tensor, received into
                 spm.state_send(got * 10, info["prev"], grp)
             info["t"] = t.tolist()
         ret[rank] = info
