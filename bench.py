@@ -18,7 +18,8 @@ Prints ONE JSON line (metric = fwd+bwd tokens/s) that also carries
   other_configs -- forward+backward times of the other benchmark configurations
                   (0: fp32; 1: single pass and as 8 chunks through lasp_fuse and
                   lasp_fuse_parallel; 3: one chunk with incoming KV; 4: 1M tokens as
-                  64 chunks), each with tokens/s and canonical TFLOP/s.
+                  64 chunks, with and without decay), each with tokens/s and canonical
+                  TFLOP/s, each timed after 100 ms of the same work.
 
 Order of the run: the other configurations, then a settling phase (--settle-ms, default 150 ms
 of the headline step, untimed), then the W warm-up steps and the K timed steps.  The settling
@@ -139,10 +140,17 @@ def cpu_baseline():
     return out
 
 
-def gpu_time(fn, iters, warm=3):
+def gpu_time(fn, iters, warm=3, settle_ms=100.0):
+    """Mean wall time of `fn` in ms over `iters` back-to-back calls, after `warm` first calls and
+    `settle_ms` of the same work (the part's clocks settle some tens of ms after the load changes)."""
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < settle_ms:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(iters):
         fn()

@@ -972,17 +972,23 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
+// skip_seg: the segment whose own state nothing reads (-1: none); its workgroups leave at once
+template <class E, bool REV, int MODE>
+int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
+                          hipStream_t st) {
+  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_STATE, st);
+  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
+                                                               skip_seg);
+  return (int)hipGetLastError();
+}
+
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
 // segment it visits last (whose own state feeds nothing else) is skipped.
 template <class E, bool REV, int MODE>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
                  bool carry_wanted, hipStream_t st) {
-  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
-  const int skip_seg = carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1);
-  ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
-                                                      skip_seg);
-  return (int)hipGetLastError();
+  return launch_state_skipping<E, REV, MODE>(y, z, s, states, g, carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1), st);
 }
 
 template <class E, int MODE>
@@ -1007,17 +1013,6 @@ int launch_fused_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
                                                          (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                          a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
                                                          (elem16_t *)a.dk, (elem16_t *)a.dv, g);
-  return (int)hipGetLastError();
-}
-
-// skip_seg: the segment whose own state nothing reads (-1: none)
-template <class E, bool REV, int MODE>
-int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
-                          hipStream_t st) {
-  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
-  ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
-                                                               skip_seg);
   return (int)hipGetLastError();
 }
 
