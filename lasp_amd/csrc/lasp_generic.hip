@@ -318,12 +318,34 @@ generic_bwd_dkdv(const T *__restrict__ Q, const T *__restrict__ K, const T *__re
 }
 
 // ------------------------------------------------------------------ segment scan
+// W consecutive columns of the stored (sd x se) state per thread (the carries are d x e).  W = 4
+// moves 16 bytes per lane and needs se % 4 == 0, e % 4 == 0 and 16-byte aligned states.
+template <int W>
+struct ScanVec {
+  float v[W];
+  __device__ void load(const float *p) {
+    if constexpr (W == 4) {
+      const float4 t = *reinterpret_cast<const float4 *>(p);
+      v[0] = t.x, v[1] = t.y, v[2] = t.z, v[3] = t.w;
+    } else {
+      v[0] = *p;
+    }
+  }
+  __device__ void store(float *p) const {
+    if constexpr (W == 4) {
+      *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      *p = v[0];
+    }
+  }
+};
+
+template <int W>
 __global__ void __launch_bounds__(256)
 segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *carry_out,
                     const float *__restrict__ S, Geom g, int reverse) {
-  // one thread per element of the stored (sd x se) state; the carries are d x e
   const int64_t sde = (int64_t)g.sd * g.se;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * W;
   const int64_t total = (int64_t)g.b * g.h * sde;
   if (idx >= total) return;
   const int bh = (int)(idx / sde);
@@ -332,33 +354,49 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   const bool in_carry = row < g.d && col < g.e;  // the padding of a stored state stays zero
   const int64_t cidx = ((int64_t)bh * g.d + row) * g.e + col;
   const float s = S[bh % g.h];
-  float run = (carry_in && in_carry) ? carry_in[cidx] : 0.f;
+  ScanVec<W> run;
+#pragma unroll
+  for (int w = 0; w < W; ++w) run.v[w] = (carry_in && in_carry) ? carry_in[cidx + w] : 0.f;
   float *p = states + (int64_t)bh * g.n_seg * sde + el;
   const float full = expf(-s * (float)g.seg_len);
   const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
   const float tail = expf(-s * (float)last_len);
-  // The loads do not depend on the recurrence: fetch a batch of segment states, then run
-  // the serial chain over the batch (forward: segments ascending; reverse: descending).
+  // The loads do not depend on the recurrence: a batch of segment states is fetched while the
+  // serial chain runs over the batch before it (forward: segments ascending; reverse: descending).
   constexpr int BATCH = 8;
-  for (int done = 0; done < g.n_seg; done += BATCH) {
-    float local[BATCH];
+  auto fetch = [&](int done, ScanVec<W> (&local)[BATCH]) {
 #pragma unroll
     for (int u = 0; u < BATCH; ++u) {
-      const int k = done + u;
+      const int k = done + u < g.n_seg ? done + u : g.n_seg - 1;  // past the end: a harmless repeat
       const int sg = reverse ? g.n_seg - 1 - k : k;
-      local[u] = k < g.n_seg ? p[(int64_t)sg * sde] : 0.f;
+      local[u].load(p + (int64_t)sg * sde);
     }
+  };
+  ScanVec<W> cur[BATCH], nxt[BATCH];
+  fetch(0, cur);
+  for (int done = 0; done < g.n_seg; done += BATCH) {
+    const bool more = done + BATCH < g.n_seg;
+    if (more) fetch(done + BATCH, nxt);
 #pragma unroll
     for (int u = 0; u < BATCH; ++u) {
       const int k = done + u;
       if (k < g.n_seg) {
         const int sg = reverse ? g.n_seg - 1 - k : k;
-        p[(int64_t)sg * sde] = run;
-        run = fmaf(sg == g.n_seg - 1 ? tail : full, run, local[u]);
+        run.store(p + (int64_t)sg * sde);
+        const float f = sg == g.n_seg - 1 ? tail : full;
+#pragma unroll
+        for (int w = 0; w < W; ++w) run.v[w] = fmaf(f, run.v[w], cur[u].v[w]);
       }
     }
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < BATCH; ++u) cur[u] = nxt[u];
+    }
   }
-  if (carry_out && in_carry) carry_out[cidx] = run;
+  if (carry_out && in_carry) {
+#pragma unroll
+    for (int w = 0; w < W; ++w) carry_out[cidx + w] = run.v[w];
+  }
 }
 
 // the largest dynamic LDS any kernel of this family asks for (generic_bwd_dkdv at d = e = 128)
@@ -437,9 +475,14 @@ int bwd_t(const BwdArgs &a, const Geom &g, hipStream_t st) {
 int launch_segment_scan(float *states, const float *carry_in, float *carry_out, const float *s,
                         const Geom &g, int reverse, hipStream_t st) {
   const int64_t total = (int64_t)g.b * g.h * g.sd * g.se;
-  const unsigned grid = (unsigned)((total + 255) / 256);
+  const bool wide = g.se % 4 == 0 && g.e % 4 == 0 && (uintptr_t)states % 16 == 0;
+  const int64_t threads = wide ? total / 4 : total;
+  const unsigned grid = (unsigned)((threads + 255) / 256);
   ProfScope prof(KC_SCAN, st);
-  segment_scan_kernel<<<grid, 256, 0, st>>>(states, carry_in, carry_out, s, g, reverse);
+  if (wide)
+    segment_scan_kernel<4><<<grid, 256, 0, st>>>(states, carry_in, carry_out, s, g, reverse);
+  else
+    segment_scan_kernel<1><<<grid, 256, 0, st>>>(states, carry_in, carry_out, s, g, reverse);
   return (int)hipGetLastError();
 }
 

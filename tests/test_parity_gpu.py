@@ -67,6 +67,7 @@ def test_library_loaded_and_path_selection(gpu_device):
 @pytest.mark.parametrize("shape", [
     (1, 2, 64, 32, 32, 0), (2, 3, 200, 64, 32, 0), (1, 2, 7, 16, 48, 0),
     (1, 2, 1024, 128, 96, 256), (1, 3, 777, 128, 64, 256), (1, 1, 33, 8, 8, 0), (1, 2, 40, 96, 128, 0),
+    (1, 2, 300, 24, 30, 64), (2, 1, 700, 17, 5, 128),   # widths that are no multiples of 4: the scan goes element by element
 ])
 def test_generic_fp32_small(gpu_device, shape, state):
     b, h, n, d, e, seg = shape
