@@ -48,8 +48,12 @@ def test_plan_defaults_and_overrides(lib):
 
     # headline shape: 16 (b,h) pairs -> 32 segments of 2048 tokens = 512 workgroups
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16) == (2048, 32, 16 * 32 * 128 * 128 * 4)
-    # short chunk: never below 256 tokens per segment
+    # short chunk: 256 tokens per segment at least ...
     assert _abi.plan(1, 16, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
+    # ... or 192 where even the backward's 3 workgroups per segment leave the chip under-filled
+    assert _abi.plan(1, 12, 2048, 128, 128, torch.bfloat16)[:2] == (192, 11)
+    assert _abi.plan(1, 2, 8192, 128, 128, torch.bfloat16)[:2] == (256, 32)   # not for one or two (b, h) pairs
+    assert _abi.plan(1, 12, 768, 128, 128, torch.bfloat16)[:2] == (256, 3)    # nor where one launch does the chunk
     # 8 segments of 256 would give the backward 3 * 24 * 8 = 576 workgroups, a few more than fit at once:
     # 7 segments of 320 (the last one 128) keep it to one round
     assert _abi.plan(2, 12, 2048, 128, 128, torch.bfloat16)[:2] == (320, 7)
