@@ -345,6 +345,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip the other configurations (profiling runs)")
     ap.add_argument("--settle-ms", type=float, default=150.0,
                     help="run the headline step untimed for this long before the warm-up steps (see the module docstring)")
+    ap.add_argument("--chain-only", action="store_true",
+                    help="run only configuration 1's 8-chunk chain through lasp_fuse and print its time (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -358,6 +360,18 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.chain_only:
+        b, h, n, chunks = 2, 12, 16384, 8
+        parts = split_chunks(device_inputs(dev, b, h, n, D, torch.bfloat16, 11, 1.0), chunks)
+        KV = torch.empty(b, h, D, D, device=dev)
+        lasp_amd.initialize_lasp(1, chunks)
+        ms = gpu_time(chain_step(lasp_amd, lasp_amd.lasp_fuse, parts, slopes(h).to(dev), KV, torch.empty_like(KV)),
+                      args.steps, warm=args.warmup, settle_ms=args.settle_ms)
+        lasp_amd.destroy_parallel_groups()
+        print(json.dumps({"workload": "config 1 as 8 chunks of 2048 tokens through lasp_fuse (loopback), forward + backward",
+                          "ms_per_step": ms, "steps": args.steps, "chunk_plan": _abi.plan(b, h, n // chunks, D, D, torch.bfloat16)[:2]}))
+        return
 
     # the headline inputs are made (on the host, seeded) before anything runs on the GPU, so that no idle
     # stretch separates the other configurations from the headline's warm-up
