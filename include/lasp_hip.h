@@ -68,6 +68,7 @@ extern "C" {
 #define LASP_E_WORKSPACE (-5)/* workspace missing or too small */
 #define LASP_E_ALIGN (-6)    /* a pointer is not aligned as the tensor contract asks */
 #define LASP_E_DEVICE (-7)   /* q is not device memory of the calling thread's current device */
+#define LASP_E_ALIAS (-8)    /* an outgoing state overlaps the incoming one where that is not supported */
 
 /* Which kernel family a shape/dtype is served by (lasp_kernel_path). */
 #define LASP_PATH_GENERIC 0 /* fp32-FMA kernels: any dtype, any n, d,e <= 128 */
@@ -106,10 +107,26 @@ int lasp_plan(int b, int h, int64_t n, int d, int e, int dtype, int seg_len_or_0
 int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype);
 
 /*
+ * Whether a call with this shape and seg_len (0 = default plan) may update its state in place:
+ * kv_out == kv_in in lasp_chunk_fwd (backward = 0), dkv_out == dkv_in in lasp_chunk_bwd
+ * (backward = 1).  Returns 1 or 0, or a negative LASP_E_*.  The pre-pass / scan / sweep kernels
+ * read the incoming state and write the outgoing one from the same thread, in that order, so
+ * there it is 1.  Where the sweeps themselves combine the states (LASP_PATH_MFMA_FUSED, and chunks
+ * of at most 4 segments on the 16-bit kernels) several workgroups read the incoming state and
+ * another one writes the outgoing state when it is done, with nothing ordering the two: it is 0
+ * unless a single workgroup does both (forward with one segment).  The reference updates in place
+ * (lasp/lasp_fuse.py:126-127,352-353); a caller that wants that where this returns 0 passes a
+ * copy of the incoming state as kv_in / dkv_in.
+ */
+int lasp_inplace_ok(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, int backward);
+
+/*
  * Forward:  O = ((Q K^T) (.) M) V + diag(l^i) Q KV_in,   M_ij = l^(i-j) [j <= i]
  *           KV_out = l^n KV_in + sum_j l^(n-j) k_j^T v_j              (l = exp(-s_h))
  * kv_in  NULL = zero incoming state.  kv_out NULL = state not wanted.
- * kv_out may alias kv_in (in-place update, as lasp/lasp_fuse.py:126-127).
+ * kv_out may be the same buffer as kv_in (in-place update, as lasp/lasp_fuse.py:126-127) where
+ * lasp_inplace_ok says so; the call returns LASP_E_ALIAS where it does not, and for buffers
+ * that overlap without being the same.
  * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds per-segment states (opaque:
  * the state entering each segment, or with few segments each segment's own contribution), which
  * lasp_chunk_bwd accepts as `kv_seg_states` -- for the same inputs, seg_len and kv_in -- to skip
@@ -149,8 +166,8 @@ int lasp_chunk_fwd_static(const void *q, const void *k, const void *v, const flo
  *   dK_j = sum_{i>=j} l^(i-j) (dO_i . v_j) q_i + l^(n-j) v_j DKV_in^T
  *   dV_j = sum_{i>=j} l^(i-j) (q_i . k_j) dO_i + l^(n-j) k_j DKV_in
  *   DKV_out = l^n DKV_in + sum_i l^i q_i^T dO_i                  (= dL/dKV_in)
- * kv_in / dkv_in NULL = zero.  dkv_out NULL = not wanted; may alias dkv_in
- * (lasp/lasp_fuse.py:352-353).
+ * kv_in / dkv_in NULL = zero.  dkv_out NULL = not wanted; may be the same buffer as dkv_in
+ * (lasp/lasp_fuse.py:352-353) under the same rule as kv_out / kv_in in the forward.
  * kv_seg_states: the array lasp_chunk_fwd left in `seg_states` for the same
  * inputs, seg_len and kv_in, or NULL to recompute it (then `workspace` must
  * hold 2 * state_bytes, else 1 * state_bytes).

@@ -56,6 +56,8 @@ def load() -> ctypes.CDLL:
                               ctypes.POINTER(_c_int), ctypes.POINTER(_c_int), ctypes.POINTER(_c_size)]
     lib.lasp_kernel_path.restype = _c_int
     lib.lasp_kernel_path.argtypes = [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int]
+    lib.lasp_inplace_ok.restype = _c_int
+    lib.lasp_inplace_ok.argtypes = [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int]
     lib.lasp_chunk_fwd.restype = _c_int
     lib.lasp_chunk_fwd.argtypes = [_c_void_p] * 8 + [_c_int, _c_int, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_void_p]
     lib.lasp_chunk_fwd_static.restype = _c_int
@@ -121,6 +123,23 @@ def kernel_path(b, h, n, d, e, dtype) -> int:
     if rc < 0:
         _raise(rc, "lasp_kernel_path")
     return rc
+
+
+@functools.lru_cache(maxsize=256)
+def inplace_ok(b, h, n, d, e, dtype, seg_len: int, backward: bool) -> bool:
+    """Whether this call may write its outgoing state over the incoming one (lasp_inplace_ok)."""
+    rc = load().lasp_inplace_ok(b, h, n, d, e, DTYPE_CODE[dtype], seg_len, int(backward))
+    if rc < 0:
+        _raise(rc, "lasp_inplace_ok")
+    return bool(rc)
+
+
+def _private_incoming(state_in, state_out, shape_key, seg_len, backward):
+    """`state_in`, or a copy of it when `state_out` is the same memory and the kernels this shape runs
+    on cannot update a state in place (the copy then plays the reference's in-place update)."""
+    if state_in is None or state_out is None or state_in.data_ptr() != state_out.data_ptr():
+        return state_in
+    return state_in if inplace_ok(*shape_key, seg_len, backward) else state_in.clone()
 
 
 KERNEL_CLASSES = ("apply", "state", "scan", "generic", "bwd3", "fused")
@@ -199,6 +218,7 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     if not fused:
         seg_len, n_seg, state_bytes = plan(b, h, n, d, e, q.dtype, seg_len)
     with _on_device(dev):
+        kv_in = _private_incoming(kv_in, kv_out, (b, h, n, d, e, q.dtype), seg_len, False)
         o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
         states = None
         if not fused and (n_seg > 1 or kv_in is not None or kv_out is not None):
@@ -266,6 +286,7 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
                             f"chunk_fwd returned for this shape, got {kv_seg_states.dtype} "
                             f"{tuple(kv_seg_states.shape)}")
     with _on_device(dev):
+        dkv_in = _private_incoming(dkv_in, dkv_out, (b, h, n, d, e, q.dtype), 0 if fused else seg_len, True)
         dq = torch.empty_like(q)
         dk = torch.empty_like(k)
         dv = torch.empty_like(v)

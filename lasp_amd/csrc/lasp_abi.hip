@@ -207,6 +207,36 @@ int check_device(const char *call, const void *q) {
   return 0;
 }
 
+// In-place state update (out == in).  The scan kernel reads the incoming carry and writes the
+// outgoing one from the same thread, so the pre-pass / scan / sweep path takes it.  On the paths
+// where the sweeps combine the states themselves every workgroup of a (b, h) reads the incoming
+// state when it starts and one of them writes the outgoing state when it ends; nothing orders a
+// late starter against an early finisher, so in place is only safe when one workgroup does both.
+bool inplace_ok(const Geom &g, bool backward) {
+  if (!g.fused && !g.combine) return true;
+  return !backward && g.n_seg == 1;  // backward: the dV workgroup writes what the dK workgroup reads
+}
+
+// `in` and `out` are states of `bytes` bytes each.
+int check_alias(const char *call, const char *what, const float *in, const float *out, size_t bytes, const Geom &g,
+                bool backward) {
+  if (!in || !out) return 0;
+  const uintptr_t a = (uintptr_t)in, b = (uintptr_t)out;
+  if (a + bytes <= b || b + bytes <= a) return 0;  // disjoint
+  if (a != b) {
+    set_error("%s: %s_out = %p overlaps %s_in = %p without being the same buffer", call, what, (const void *)out,
+              what, (const void *)in);
+    return LASP_E_ALIAS;
+  }
+  if (!inplace_ok(g, backward)) {
+    set_error("%s: %s_out is %s_in, but this shape runs kernels in which one workgroup writes the outgoing state "
+              "while others may still have to read the incoming one (see lasp_inplace_ok); pass a copy as %s_in",
+              call, what, what, what);
+    return LASP_E_ALIAS;
+  }
+  return 0;
+}
+
 // ---- segment-state scratch owned by the library (lasp_chunk_fwd_static) ------------------------
 // Lives in the code object: every device the library runs on holds its own copy, at its own
 // address, until the process ends.  In host code the array's name is only a handle for
@@ -342,10 +372,18 @@ int lasp_kernel_path(int b, int h, int64_t n, int d, int e, int dtype) {
   return (mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype)) ? LASP_PATH_MFMA : LASP_PATH_GENERIC;
 }
 
+int lasp_inplace_ok(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, int backward) {
+  Geom g;
+  int rc = make_geom(b, h, n, d, e, dtype, seg_len, &g);
+  if (rc) return rc;
+  return inplace_ok(g, backward != 0) ? 1 : 0;
+}
+
 static int chunk_fwd_impl(const char *me, const void *q, const void *k, const void *v, const float *s,
                           const float *kv_in, float *kv_out, void *o, float *seg_states, const Geom &g,
                           int dtype, void *stream) {
   int rc;
+  if ((rc = check_alias(me, "kv", kv_in, kv_out, sizeof(float) * (size_t)g.b * g.h * g.d * g.e, g, false))) return rc;
   if ((rc = check_aligned(me, "q", q, 16)) || (rc = check_aligned(me, "k", k, 16)) ||
       (rc = check_aligned(me, "v", v, 16)) || (rc = check_aligned(me, "o", o, 16)) ||
       (rc = check_aligned(me, "s", s, 4)) || (rc = check_aligned(me, "kv_in", kv_in, 4)) ||
@@ -425,6 +463,7 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s, 
     return LASP_E_WORKSPACE;
   }
   const char *me = "lasp_chunk_bwd";
+  if ((rc = check_alias(me, "dkv", dkv_in, dkv_out, sizeof(float) * (size_t)b * h * d * e, g, true))) return rc;
   if ((rc = check_aligned(me, "q", q, 16)) || (rc = check_aligned(me, "k", k, 16)) ||
       (rc = check_aligned(me, "v", v, 16)) || (rc = check_aligned(me, "do", d_o, 16)) ||
       (rc = check_aligned(me, "dq", dq, 16)) || (rc = check_aligned(me, "dk", dk, 16)) ||

@@ -114,6 +114,34 @@ def test_null_and_workspace_errors_need_no_gpu(lib):
     assert rc == -5 and b"workspace" in lib.lasp_last_error()
 
 
+def test_in_place_state_update_rules(lib):
+    """Out == in is taken where one thread (the scan) or one workgroup (a single segment, forward)
+    reads the incoming state and writes the outgoing one; elsewhere, and for buffers that merely
+    overlap, the call is refused before anything is launched."""
+    from lasp_amd import _abi
+
+    bf, f32 = torch.bfloat16, torch.float32
+    assert _abi.inplace_ok(2, 12, 2048, 128, 128, bf, 0, False) and _abi.inplace_ok(2, 12, 2048, 128, 128, bf, 0, True)
+    assert _abi.kernel_path(1, 2, 512, 128, 128, bf) == _abi.PATH_MFMA_FUSED      # two segments, one launch
+    assert not _abi.inplace_ok(1, 2, 512, 128, 128, bf, 0, False) and not _abi.inplace_ok(1, 2, 512, 128, 128, bf, 0, True)
+    assert _abi.inplace_ok(1, 2, 512, 128, 128, bf, 64, False)                    # explicit seg_len: 8 segments, scan
+    assert not _abi.inplace_ok(2, 12, 1024, 128, 128, bf, 256, False)             # 4 segments: the sweeps gather
+    assert _abi.inplace_ok(8, 128, 4096, 128, 128, bf, 0, False)                  # one segment, one workgroup
+    assert not _abi.inplace_ok(8, 128, 4096, 128, 128, bf, 0, True)               # dV writes what dK reads
+    assert _abi.inplace_ok(1, 2, 512, 128, 128, f32, 0, False) and _abi.inplace_ok(1, 2, 512, 128, 128, f32, 0, True)
+
+    ok, kv = ctypes.c_void_p(4096), ctypes.c_void_p(1 << 20)
+    fwd = lambda n, seg, kv_in, kv_out: lib.lasp_chunk_fwd(ok, ok, ok, ok, kv_in, kv_out, ok, ok, 1, 2, n, 128, 128,
+                                                           1, seg, None)
+    assert fwd(512, 0, kv, kv) == -8 and b"lasp_inplace_ok" in lib.lasp_last_error()
+    assert fwd(512, 64, kv, ctypes.c_void_p((1 << 20) + 64)) == -8 and b"overlaps" in lib.lasp_last_error()
+    assert fwd(512, 64, kv, kv) == -7   # accepted as far as aliasing goes: the next check (device) is what stops it here
+    bwd = lambda n, seg: lib.lasp_chunk_bwd(ok, ok, ok, ok, ok, None, kv, ok, ok, ok, kv, None, ok, 1 << 30, 1, 2, n,
+                                            128, 128, 1, seg, None)
+    assert bwd(512, 0) == -8 and b"dkv_out is dkv_in" in lib.lasp_last_error()
+    assert bwd(512, 64) == -7
+
+
 def test_alignment_and_device_errors_need_no_gpu(lib):
     """A misaligned tensor or state pointer is LASP_E_ALIGN; a pointer HIP does not know as memory of
     the current device is LASP_E_DEVICE.  Both are reported before anything is launched."""

@@ -231,11 +231,14 @@ def test_operator_chain_in_a_graph(gpu_device, op_name):
     assert O.rel_err(torch.cat(eager[chunks::3], 2).cpu(), ref["dq"]) <= 2e-2
 
 
+@pytest.mark.parametrize("n", [512, 1024, 4096])   # bf16, e = 128: one launch / sweeps that gather 4 segments / scan
 @pytest.mark.parametrize("dtype,e", [(torch.bfloat16, 128), (torch.float32, 128), (torch.bfloat16, 64)])
-def test_launch_shims_against_oracle(gpu_device, dtype, e):
+def test_launch_shims_against_oracle(gpu_device, dtype, e, n):
     """lasp_fuse.lasp_forward/lasp_backward (states in place) and the lasp_fuse_parallel pair
     (new state tensors, segment-state cache handed from forward to backward) on one chunk with
-    incoming KV and dKV (lasp/lasp_fuse.py:356-475, lasp/lasp_fuse_parallel.py:833-1070)."""
+    incoming KV and dKV (lasp/lasp_fuse.py:356-475, lasp/lasp_fuse_parallel.py:833-1070).
+    In place works on every kernel path: where the kernels cannot update a state in place the
+    binding hands them a copy of the incoming one."""
     import importlib
 
     from tests.helpers import TOL, check, oracle
@@ -243,7 +246,7 @@ def test_launch_shims_against_oracle(gpu_device, dtype, e):
     LF = importlib.import_module("lasp_amd.lasp_fuse")
     LP = importlib.import_module("lasp_amd.lasp_fuse_parallel")
     dev = gpu_device
-    b, h, n, d = 1, 4, 1024, 128
+    b, h, d = 1, 4, 128
     s = O.slopes_baseline(h)
     inp = make_inputs(b, h, n, d, e, dtype, seed=31, scale=d ** -0.5, state=True, device=dev)
     ref = oracle(inp, s)
