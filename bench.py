@@ -21,8 +21,10 @@ Prints ONE JSON line (metric = fwd+bwd tokens/s) that also carries
                   64 chunks, with and without decay), each with tokens/s and canonical
                   TFLOP/s, each timed after 100 ms of the same work.
 
-Order of the run: the other configurations, then a settling phase (--settle-ms, default 150 ms
-of the headline step, untimed), then the W warm-up steps and the K timed steps.  The settling
+Order of the run: the other configurations; W warm-up and K timed steps of the headline step as they
+come (`ms_per_step_unsettled`); a settling phase (--settle-ms, default 150 ms of the headline step,
+untimed); then the W warm-up steps and the K timed steps behind `value` (`warmup_effective` counts
+every untimed step before them).  The settling
 phase is there because the part answers every change of load with a power-management transient:
 for about 30 ms after these kernels start -- from idle or straight after other GPU work -- every
 kernel runs 5-30 % slower, back to back with no gaps between them, and then settles.  A training
@@ -88,6 +90,54 @@ def read_traffic_profile(path=HBM_PROFILE):
     for m in re.finditer(r"^traffic\s+(\S+)\s+fetch_kib=([0-9.]+)\s+write_kib=([0-9.]+)", text, flags=re.M):
         kernels[m.group(1)] = int((float(m.group(2)) * f_scale + float(m.group(3)) * w_scale) * 1024)
     return {"seg_len": int(plan.group(1)), "n_seg": int(plan.group(2)), "kernels": kernels}
+
+
+CEILING_PROFILE = os.path.join(ROOT, "profiles", "stream_probe_hbm_ceiling.txt")
+
+
+def read_ceiling_profile(path=CEILING_PROFILE):
+    """{"4:3": GB/s, ...} from the committed summary of `bench.py --stream-probe` (lines `ceiling mix=R:W gbs=...`),
+    or None if there is no such file."""
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    found = {m.group(1): float(m.group(2)) for m in re.finditer(r"^ceiling\s+mix=(\d+:\d+)\s+gbs=([0-9.]+)", text, flags=re.M)}
+    return found or None
+
+
+def stream_probe(dev, mib_each, iters):
+    """What the memory system sustains for the sweeps' access pattern with no arithmetic: R read and W write
+    streams of `mib_each` MiB through lasp_stream_probe, best grid of a small sweep, next to a plain device copy."""
+    from lasp_amd import _abi
+
+    n = mib_each << 20
+    bufs = [torch.empty(n, dtype=torch.uint8, device=dev).fill_(1) for _ in range(10)]
+    rows = []
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(iters):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / iters
+
+    ms = timed(lambda: bufs[1].copy_(bufs[0]))
+    rows.append({"mix": "copy_", "reads": 1, "writes": 1, "grid": None, "us": ms * 1e3, "gbs": 2 * n / ms / 1e6})
+    for r, w in ((1, 0), (2, 0), (4, 0), (0, 1), (1, 1), (3, 1), (4, 3), (7, 3)):
+        best = None
+        for grid in (512, 1024, 2048, 4096, 8192):
+            ms = timed(lambda: _abi.stream_probe(bufs[:r], bufs[r:r + w], grid))
+            if best is None or ms < best[1]:
+                best = (grid, ms)
+        rows.append({"mix": f"{r}:{w}", "reads": r, "writes": w, "grid": best[0], "us": best[1] * 1e3,
+                     "gbs": (r + w) * n / best[1] / 1e6})
+    return rows
 
 
 def cpu_cores():
@@ -347,6 +397,9 @@ def main():
                     help="run the headline step untimed for this long before the warm-up steps (see the module docstring)")
     ap.add_argument("--chain-only", action="store_true",
                     help="run only configuration 1's 8-chunk chain through lasp_fuse and print its time (profiling runs)")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="run only the streaming-bandwidth probe (read:write mixes with no arithmetic) and print its table")
+    ap.add_argument("--probe-mib", type=int, default=1024, help="size of each stream of the probe, MiB")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -360,6 +413,16 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.stream_probe:
+        rows = stream_probe(dev, args.probe_mib, 20)
+        print(f"# streaming probe: streams of {args.probe_mib} MiB each, 16 KiB pieces, 16-byte accesses, "
+              f"non-temporal stores; best of grids 512..8192; {torch.cuda.get_device_name(dev)}")
+        for r in rows:
+            print(f"ceiling mix={r['mix']} gbs={r['gbs']:.0f}  # footprint {(r['reads'] + r['writes']) * args.probe_mib} MiB, "
+                  f"{r['us']:.1f} us per launch, grid {r['grid']}")
+        print(json.dumps({"stream_probe": rows, "mib_each": args.probe_mib}))
+        return
 
     if args.chain_only:
         b, h, n, chunks = 2, 12, 16384, 8
@@ -400,6 +463,15 @@ def main():
     for _ in range(3):  # first calls: library load, kernel attributes, allocator growth
         step()
     torch.cuda.synchronize()
+    # the driver's regime as it stands: W warm-up steps, then K timed steps, before any settling
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step_unsettled = (time.perf_counter() - t0) / args.steps * 1e3
     settle_steps = 0
     t0 = time.perf_counter()
     while (time.perf_counter() - t0) * 1e3 < args.settle_ms:
@@ -437,11 +509,20 @@ def main():
     profile = read_traffic_profile()
     same_plan = profile is not None and (profile["seg_len"], profile["n_seg"]) == (seg_len, n_seg)
 
-    def roof(kernel, cls, alg_bytes):
+    ceilings = read_ceiling_profile()
+
+    def roof(kernel, cls, alg_bytes, mix):
         ms, cnt = prof[cls]
         avg_ms = ms / max(cnt, 1)
         achieved = alg_bytes / (avg_ms * 1e-3) / 1e9
+        extra = {}
+        if ceilings and mix in ceilings:
+            # what a kernel that only streams this read:write mix reached on this part (profiles/)
+            extra = {"measured_ceiling": ceilings[mix], "measured_ceiling_mix": mix,
+                     "frac_of_measured_ceiling": achieved / ceilings[mix],
+                     "measured_ceiling_source": os.path.relpath(CEILING_PROFILE, ROOT)}
         return {
+            **extra,
             "kernel": kernel, "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": profile["kernels"].get(kernel) if same_plan else None,
@@ -461,7 +542,11 @@ def main():
         "warmup": args.warmup,
         "settle_ms": args.settle_ms,
         "settle_steps": settle_steps,
+        # untimed steps that ran before the timed ones: first calls, the unsettled measurement (W + K), settling, W
+        "warmup_effective": 3 + args.warmup + args.steps + settle_steps + args.warmup,
         "ms_per_step": ms_step,
+        # K steps timed straight after 3 first calls and W warm-up steps, before the settling phase
+        "ms_per_step_unsettled": ms_step_unsettled,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -482,9 +567,9 @@ def main():
         "kernel_ms": {name: {"total_ms": ms, "launches": cnt} for name, (ms, cnt) in prof.items() if cnt},
         "kernel_sum_ms_per_step": kernel_sum_ms,
         # dominant kernel: la_bwd3 (one launch = the whole backward sweep: reads Q,K,V,dO, writes dQ,dK,dV)
-        "roofline": roof("la_bwd3", "bwd3", BYTES_BWD_PER_TH * th),
+        "roofline": roof("la_bwd3", "bwd3", BYTES_BWD_PER_TH * th, "4:3"),
         # second kernel: la_apply (one launch = the forward sweep: reads Q,K,V, writes O)
-        "roofline_fwd": roof("la_apply", "apply", BYTES_FWD_PER_TH * th),
+        "roofline_fwd": roof("la_apply", "apply", BYTES_FWD_PER_TH * th, "3:1"),
     }
     if extras is not None:
         out["other_configs"] = extras

@@ -128,7 +128,8 @@ int lasp_inplace_ok(int b, int h, int64_t n, int d, int e, int dtype, int seg_le
  * lasp_inplace_ok says so; the call returns LASP_E_ALIAS where it does not, and for buffers
  * that overlap without being the same.
  * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds per-segment states (opaque:
- * the state entering each segment, or with few segments each segment's own contribution), which
+ * the state entering each segment; each segment's own contribution with few segments, and for
+ * heads whose decay wipes a state within one segment, which the scan leaves out), which
  * lasp_chunk_bwd accepts as `kv_seg_states` -- for the same inputs, seg_len and kv_in -- to skip
  * recomputing them.  It may be NULL when n_seg == 1 and kv_in == NULL and kv_out == NULL, and on
  * LASP_PATH_MFMA_FUSED.
@@ -150,6 +151,9 @@ int lasp_chunk_fwd(const void *q, const void *k, const void *v, const float *s,
  * path) must fit, i.e. at most 512 states on the MFMA path -- the headline shape
  * b=1 h=16 n=65536 with the default seg_len just fits; a larger call returns
  * LASP_E_WORKSPACE (a longer seg_len lowers n_seg).
+ * The first call on a device looks the scratch's device address up (hipGetSymbolAddress, which
+ * may also make the runtime load the library's code object on that device): make one call per
+ * device before entering a region that must not do that, e.g. before starting a graph capture.
  * All calls on one GPU share that GPU's scratch: two calls whose work overlaps in time
  * on one GPU (different streams, or different threads) race on it.  The states are not
  * returned, so a backward of the same chunk recomputes them (kv_seg_states = NULL).
@@ -199,6 +203,19 @@ int lasp_chunk_bwd(const void *q, const void *k, const void *v, const float *s,
 #define LASP_KC_FUSED 5   /* la_fused_fwd / la_fused_bwd: a short chunk in one launch */
 int lasp_profile_begin(int max_launches);
 int lasp_profile_end(double *ms_per_class, int *launches_per_class);
+
+/*
+ * Second measurement hook (no counterpart in the reference): one launch of a kernel that only
+ * streams -- n_rd read streams and n_wr write streams of bytes_each bytes (a multiple of 16384),
+ * walked in 16 KiB pieces with 16-byte accesses and non-temporal stores, the way the sweeps walk
+ * their token blocks, by `grid` workgroups of 256 threads.  Built mixes (reads:writes): 1:0, 2:0,
+ * 4:0, 0:1, 1:1, 3:1 (the forward sweep's), 4:3 (the backward sweep's), 7:3 (what the backward
+ * sweep really moves).  rd / wr are HOST arrays of device pointers, each 16-byte aligned.  The
+ * caller times it (events on `stream`); the rate it reaches is the ceiling the sweeps are
+ * compared with beside the published HBM peak.
+ */
+int lasp_stream_probe(const void *const *rd, int n_rd, void *const *wr, int n_wr, size_t bytes_each,
+                      int grid, void *stream);
 
 #ifdef __cplusplus
 }

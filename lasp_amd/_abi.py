@@ -68,6 +68,9 @@ def load() -> ctypes.CDLL:
     lib.lasp_profile_begin.argtypes = [_c_int]
     lib.lasp_profile_end.restype = _c_int
     lib.lasp_profile_end.argtypes = [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(_c_int)]
+    lib.lasp_stream_probe.restype = _c_int
+    lib.lasp_stream_probe.argtypes = [ctypes.POINTER(_c_void_p), _c_int, ctypes.POINTER(_c_void_p), _c_int, _c_size,
+                                      _c_int, _c_void_p]
     if lib.lasp_abi_version() != 1:
         raise LaspError(f"ABI version mismatch: library reports {lib.lasp_abi_version()}, binding expects 1")
     _lib = lib
@@ -160,6 +163,22 @@ def profile_end() -> dict:
     if rc:
         _raise(rc, "lasp_profile_end")
     return {name: (ms[i], cnt[i]) for i, name in enumerate(KERNEL_CLASSES)}
+
+
+def stream_probe(reads, writes, grid: int) -> None:
+    """Enqueues one launch of the streaming probe (lasp_stream_probe) on torch's current stream: every tensor
+    of `reads` is read once and every tensor of `writes` written once; all must have the same byte size."""
+    lib = load()
+    sizes = {t.numel() * t.element_size() for t in (*reads, *writes)}
+    if len(sizes) != 1:
+        raise LaspError(f"the probe's streams must all have the same size, got {sorted(sizes)}")
+    dev = _check_dev(*reads, *writes)
+    rd = (_c_void_p * max(len(reads), 1))(*[t.data_ptr() for t in reads])
+    wr = (_c_void_p * max(len(writes), 1))(*[t.data_ptr() for t in writes])
+    rc = lib.lasp_stream_probe(rd, len(reads), wr, len(writes), sizes.pop(), grid,
+                               torch.cuda.current_stream(dev).cuda_stream)
+    if rc:
+        _raise(rc, "lasp_stream_probe")
 
 
 def _shapes(q, k, v):

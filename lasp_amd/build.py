@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblasp_hip.so")
-SOURCES = ["lasp_abi.hip", "lasp_generic.hip", "lasp_mfma.hip", "lasp_mfma_f32.hip"]
+SOURCES = ["lasp_abi.hip", "lasp_generic.hip", "lasp_mfma.hip", "lasp_mfma_f32.hip", "lasp_probe.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -171,6 +171,8 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   g->fused = fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg) ? 1 : 0;
   g->combine = (!g->fused && mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature &&
                 n_seg <= kCombineMaxSeg) ? 1 : 0;
+  // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
+  g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg >= 2) ? 1 : 0;
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;

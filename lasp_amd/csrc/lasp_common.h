@@ -59,7 +59,24 @@ struct Geom {
                 // generic kernels, 128 x 128 (zero beyond d, e) for the MFMA kernels
   int fused;    // the chunk is served by the single-launch kernels, which use no workspace
   int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
+  int bypass;   // the scan leaves out heads whose state dies within one segment (see state_dies_in_segment)
 };
+
+// Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels: far under the
+// 2^-24 rounding of the fp32 sums they would be added to.
+constexpr float kSkipLog2 = 64.f;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// With g.bypass set, a head whose decay over the chunk's shortest segment (the last one) is below
+// 2^-kSkipLog2 takes no part in the scan: whatever enters a segment has faded to nothing at its far
+// end, so the state entering segment j is the OWN state of the segment before it (after it, going
+// backwards) and, for the first segment visited, the chunk's incoming state.  The scan kernel
+// leaves those heads' own states in place and only forms their outgoing carry; the sweeps read the
+// neighbour's own state.  Both sides must take the same decision, hence this one function.
+__device__ __forceinline__ bool state_dies_in_segment(float slope, const Geom &g) {
+  const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
+  return g.bypass != 0 && slope * kLog2e * (float)last_len > kSkipLog2;
+}
 
 // Host-side launchers (each returns a hipError_t as int, or a negative LASP_E_*).
 struct FwdArgs {

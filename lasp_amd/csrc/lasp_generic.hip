@@ -361,6 +361,20 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   const float full = expf(-s * (float)g.seg_len);
   const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
   const float tail = expf(-s * (float)last_len);
+  if (state_dies_in_segment(s, g)) {
+    // This head's own states stay as the pre-pass wrote them (the sweeps read the neighbour's).  Only the
+    // outgoing carry is formed, from the two segments visited last: anything older has faded below 2^-64.
+    if (carry_out && in_carry) {
+      const int prev = reverse ? 1 : g.n_seg - 2, end = reverse ? 0 : g.n_seg - 1;
+      ScanVec<W> a, b;
+      a.load(p + (int64_t)prev * sde);
+      b.load(p + (int64_t)end * sde);
+      const float f = end == g.n_seg - 1 ? tail : full;
+#pragma unroll
+      for (int w = 0; w < W; ++w) carry_out[cidx + w] = fmaf(f, a.v[w], b.v[w]);
+    }
+    return;
+  }
   // The loads do not depend on the recurrence: a batch of segment states is fetched while the
   // serial chain runs over the batch before it (forward: segments ascending; reverse: descending).
   constexpr int BATCH = 8;

@@ -58,8 +58,8 @@ constexpr int OFF_YT = OFF_YN + BLK * LDN;
 constexpr int OFF_ZT = OFF_YT + F * LDT;
 constexpr int OFF_SC = OFF_ZT + F * LDT;
 constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float SKIP_LOG2 = 64.f;  // decay weights below 2^-SKIP_LOG2 are treated as zero (see la_seg_state)
+constexpr float LOG2E = kLog2e;
+constexpr float SKIP_LOG2 = kSkipLog2;  // decay weights below 2^-SKIP_LOG2 are treated as zero (see la_seg_state)
 enum Mode { M_ALIGNED = 0, M_RAGGED = 1, M_NARROW = 2 };
 // where a sweep takes the state entering its segment from (see apply_body)
 enum Source { SRC_SCANNED = 0, SRC_WALK = 1, SRC_COMBINE = 2 };
@@ -405,7 +405,24 @@ apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const
       }
     }
   } else if (SRC == SRC_SCANNED && states) {
-    add_state(states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F), F, 0.f, false);
+    // Scanned states sit at the segment's own index.  A head the scan leaves out (state_dies_in_segment)
+    // still has the pre-pass's own states there: the state entering this segment is then the own state
+    // of the segment visited before it, or the chunk's incoming state for the first one.
+    const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
+    int ld = F;
+    bool bounded = false, have = true;
+    if (state_dies_in_segment(S[sw.bh % g.h], g)) {
+      const int nb = REV ? sw.seg + 1 : sw.seg - 1;
+      if (nb < 0 || nb >= g.n_seg) {
+        have = carry_in != nullptr;
+        src = carry_in + (int64_t)sw.bh * fa * fb;  // fa x fb floats, unpadded
+        ld = NARROW ? (TRANS ? fa : fb) : F;
+        bounded = NARROW;
+      } else {
+        src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
+      }
+    }
+    if (have) add_state(src, ld, 0.f, bounded);
   }
 
   // ---- block loader: registers <- global, LDS <- registers
@@ -1035,7 +1052,7 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
   return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
-                                                          nullptr, nullptr, a.o, g, st);
+                                                          a.kv_in, nullptr, a.o, g, st);
 }
 
 template <class E, int MODE>

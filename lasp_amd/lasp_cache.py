@@ -32,11 +32,15 @@ def lasp_backward(q, k, v, s, do):
 
 
 class LaspCache(torch.autograd.Function):
-    """forward(q, k, v, s, array, KV, DKV) as lasp/lasp_cache.py:539-617."""
+    """forward(q, k, v, s, array, KV, DKV) as lasp/lasp_cache.py:539-617.
+
+    The reference receives into the caller's KV / DKV and then rebinds the name to a new tensor
+    (`KV = block_decay * KV + kv`, :562; `DKV = ...`, :609), so after a call the caller's buffers hold
+    the INCOMING states; the same here."""
 
     @staticmethod
     def forward(ctx, q, k, v, s, array, KV, DKV):
-        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, True, False)
+        return ChunkFunction.forward(ctx, q, k, v, s, KV, DKV, True, False, True)
 
     @staticmethod
     def backward(ctx, do):
@@ -49,4 +53,4 @@ lasp_cache_ = LaspCache.apply
 def lasp_cache(q, k, v, ed, array, KV, DKV):
     if q.shape[-1] <= 128:
         return lasp_cache_(q, k, v, ed, array, KV, DKV)
-    return run_sliced(q, k, v, ed, KV, DKV, True, False)
+    return run_sliced(q, k, v, ed, KV, DKV, True, False, True)

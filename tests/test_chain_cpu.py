@@ -84,16 +84,17 @@ def test_chain_choreography_equals_single_pass(op_name):
         assert O.rel_err(got, ref[name]) < tol, (op_name, name)
     _, kv1 = O.ref_chunked_fwd(q[:, :, :64], k[:, :, :64], v[:, :, :64], s, None, 64, torch.float64)
     _, kv3 = O.ref_chunked_fwd(q[:, :, :192], k[:, :, :192], v[:, :, :192], s, None, 64, torch.float64)
-    if op_name in ("lasp_fuse", "lasp_cache"):
+    if op_name == "lasp_fuse":
         # the caller's KV holds KV_out of the chunk just run; after the last chunk, of the whole sequence
         # (in-place update, lasp/lasp_fuse.py:126-127)
         assert O.rel_err(kv_after[-1], ref["kv_out"]) < 1e-12
         assert O.rel_err(kv_after[0], kv1) < 1e-12
         # after the reversed chain the caller's DKV holds dL/dKV_in of the first chunk
         assert O.rel_err(dkv_after[0], ref["dkv_out"]) < 1e-12
-    elif op_name == "lasp_fuse_parallel":
-        # the caller's buffers are left holding the INCOMING states (lasp/lasp_fuse_parallel.py:1091-1101:
-        # KV is zeroed, received into, and the outgoing state is bound to a new tensor)
+    elif op_name in ("lasp_fuse_parallel", "lasp_cache"):
+        # the caller's buffers are left holding the INCOMING states (lasp/lasp_fuse_parallel.py:1091-1101,
+        # lasp/lasp_cache.py:549-562,597-609: KV is zeroed, received into, and the outgoing state is bound
+        # to a new tensor)
         assert torch.count_nonzero(kv_after[0]) == 0
         assert O.rel_err(kv_after[1], kv1) < 1e-12
         assert O.rel_err(kv_after[-1], kv3) < 1e-12

@@ -111,7 +111,8 @@ def test_config4_million_tokens_chunk_chain(gpu_device, variant):
     """b=1 h=16 n=1048576 d=128 bf16 as 64 chunks of 16384 with KV / DKV carry.
 
     Oracle (fp32 recurrence over the whole sequence) on heads {0, 15}; the chain is
-    also compared with one single-pass launch over all 1M tokens for every head."""
+    also compared with one single-pass launch over all 1M tokens for every head, and run a second time
+    through the lasp_fuse operator with the loopback."""
     from lasp_amd import _abi
 
     dev = gpu_device
@@ -151,10 +152,45 @@ def test_config4_million_tokens_chunk_chain(gpu_device, variant):
     heads = [0, 15]
     ref = _oracle_heads(q, k, v, do, s, heads)
     _check_heads(got, ref, heads, ("o", "dq", "dk", "dv"))
-    del ref
 
     single = _fwd_bwd(q, k, v, do, s)
     torch.cuda.synchronize()
     for name in ("o", "dq", "dk", "dv"):
         for hd in range(h):  # per head: the scale of the outputs differs by orders of magnitude across slopes
             assert _rel(got[name][:, hd], single[name][:, hd]) <= TOL, (name, hd)
+    del single
+
+    # the same 64-chunk chain through the public operator (autograd + loopback state passing, one process
+    # playing every rank): heads {0, 15} against the oracle, every head against the raw-ABI chain above
+    via_op = _operator_chain(q, k, v, do, s, chunks)
+    _check_heads(via_op, ref, heads, ("o", "dq", "dk", "dv"))
+    for name in ("o", "dq", "dk", "dv"):
+        for hd in range(h):
+            assert _rel(via_op[name][:, hd], got[name][:, hd]) <= TOL, (name, hd)
+
+
+def _operator_chain(q, k, v, do, s, chunks):
+    import lasp_amd
+
+    b, h, n, d = q.shape
+    step = n // chunks
+    KV = torch.empty(b, h, d, d, device=q.device)
+    DKV = torch.empty_like(KV)
+    lasp_amd.destroy_parallel_groups()
+    lasp_amd.initialize_lasp(1, chunks)
+    outs, leaves = [], []
+    try:
+        for c in range(chunks):
+            lasp_amd.set_sequence_parallel_rank(c)
+            sl = slice(c * step, (c + 1) * step)
+            qc, kc, vc = [t[:, :, sl].clone().requires_grad_(True) for t in (q, k, v)]
+            outs.append(lasp_amd.lasp_fuse(qc, kc, vc, s, KV, DKV))
+            leaves.append((qc, kc, vc))
+        for c in reversed(range(chunks)):
+            outs[c].backward(do[:, :, c * step:(c + 1) * step])
+        torch.cuda.synchronize()
+        assert lasp_amd.loopback_pending() == []
+    finally:
+        lasp_amd.destroy_parallel_groups()
+    return dict(o=torch.cat([o.detach() for o in outs], 2), dq=torch.cat([l[0].grad for l in leaves], 2),
+                dk=torch.cat([l[1].grad for l in leaves], 2), dv=torch.cat([l[2].grad for l in leaves], 2))

@@ -55,6 +55,41 @@ def test_static_scratch_forward_matches_workspace_forward_twice(gpu_device):
         assert O.rel_err(o_st, ref_o) <= 2e-2 and O.rel_err(kv_st, ref_kv) <= 2e-2
 
 
+@pytest.mark.parametrize("shape,seg", [((1, 4, 2048, 128, 128), 256),    # pre-pass / scan / sweep: 8 segments
+                                       ((2, 3, 1536, 128, 128), 512),    # scan-less: 3 segments gathered by the sweeps
+                                       ((1, 2, 320, 128, 128), 0),       # default plan: a single launch, no states
+                                       ((1, 2, 700, 128, 64), 256)])     # narrow rows, ragged length
+def test_static_scratch_forward_allocates_nothing(gpu_device, shape, seg):
+    """After a first (warm) call -- which looks the scratch's address up and loads the kernels -- a second
+    call must leave the device's free memory and torch's allocation count where they were, and give the
+    workspace variant's bits."""
+    from lasp_amd import _abi
+
+    lib = _abi.load()
+    dev = gpu_device
+    b, h, n, d, e = shape
+    inp = make_inputs(b, h, n, d, e, torch.bfloat16, seed=74, scale=d ** -0.5, state=True, device=dev)
+    s = O.slopes_baseline(h).reshape(-1).to(dev)
+    want, _, _ = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=torch.empty_like(inp["kv"]),
+                                seg_len=seg)
+    o, kv_out = torch.empty_like(inp["v"]), torch.empty_like(inp["kv"])
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    args = (inp["q"].data_ptr(), inp["k"].data_ptr(), inp["v"].data_ptr(), s.data_ptr(), inp["kv"].data_ptr(),
+            kv_out.data_ptr(), o.data_ptr(), b, h, n, d, e, _abi.DTYPE_CODE[torch.bfloat16], seg, stream)
+    print(f"lasp_chunk_fwd_static warm call b={b} h={h} n={n} d={d} e={e} seg_len={seg}", flush=True)
+    assert lib.lasp_chunk_fwd_static(*args) == 0, lib.lasp_last_error()
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    allocs_before = torch.cuda.memory_stats(dev)["allocation.all.allocated"]
+    o.zero_()  # in place: no allocation
+    print("lasp_chunk_fwd_static second call", flush=True)
+    assert lib.lasp_chunk_fwd_static(*args) == 0, lib.lasp_last_error()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
+    assert torch.cuda.memory_stats(dev)["allocation.all.allocated"] == allocs_before
+    assert torch.equal(o, want)
+
+
 def test_static_scratch_python_wrapper_and_size_limit(gpu_device):
     from lasp_amd import _abi
 
