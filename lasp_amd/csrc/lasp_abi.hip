@@ -2,6 +2,7 @@
 // the kernel families.  Declarations and the tensor contract: include/lasp_hip.h.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include <atomic>
 
@@ -173,6 +174,10 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
                 n_seg <= kCombineMaxSeg) ? 1 : 0;
   // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
   g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg >= 2) ? 1 : 0;
+  {
+    const char *ev = getenv("LASP_WS");  // experiment switch
+    g->ws = ((!ev || atoi(ev) != 0) && mfma_eligible(d, e, dtype) && !g->fused && !g->combine) ? 1 : 0;
+  }
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;

@@ -60,11 +60,14 @@ struct Geom {
   int fused;    // the chunk is served by the single-launch kernels, which use no workspace
   int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
   int bypass;   // the scan leaves out heads whose state dies within one segment (see state_dies_in_segment)
+  int ws;       // aligned 16-bit chunks on the scan path run the wave-specialised sweeps (la_apply_ws, la_bwd3_ws)
 };
 
-// Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels: far under the
-// 2^-24 rounding of the fp32 sums they would be added to.
-constexpr float kSkipLog2 = 64.f;
+// Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels.  A state is an fp32 sum
+// whose largest terms carry weights near 1 (the tokens next to the segment's far end), so what is dropped
+// lies below the rounding of that sum itself -- and the kernels round every state to 16 bits (2^-9 for
+// bf16) before they multiply with it.
+constexpr float kSkipLog2 = 24.f;
 constexpr float kLog2e = 1.4426950408889634f;
 
 // With g.bypass set, a head whose decay over the chunk's shortest segment (the last one) is below

@@ -363,7 +363,7 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   const float tail = expf(-s * (float)last_len);
   if (state_dies_in_segment(s, g)) {
     // This head's own states stay as the pre-pass wrote them (the sweeps read the neighbour's).  Only the
-    // outgoing carry is formed, from the two segments visited last: anything older has faded below 2^-64.
+    // outgoing carry is formed, from the two segments visited last: anything older has faded below 2^-24.
     if (carry_out && in_carry) {
       const int prev = reverse ? 1 : g.n_seg - 2, end = reverse ? 0 : g.n_seg - 1;
       ScanVec<W> a, b;

@@ -794,6 +794,309 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
 }
 
 // ------------------------------------------------------------------------------
+// The sweep with the work of a block split between two groups of waves (chunk length a multiple of
+// 64, d = e = 128, state taken from the scan).  apply_body runs fill -> products -> store one after the
+// other in every wave, so a workgroup alone on a CU spends most of a block waiting for its own LDS
+// round trips; here 512 threads form one workgroup per CU:
+//   waves 0-3 ("feed"): global loads, the LDS tiles of the NEXT block (transposes and decay scaling
+//     included), the masked score tile of the current block, the coalesced output stores;
+//   waves 4-7 ("math"): own the state and the output accumulators (wave 4 + w: columns [32w, 32w + 32)):
+//     state term, intra-block term, state update, output staging.
+// The tiles are double-buffered (two sets of X, Y token-major and Y^T, Z^T feature-major, 144 384 B
+// with the score tile), and a block takes two barriers:
+//     feed: store O(t-1), score(t)    | math: state term(t)
+//   ---- barrier ----
+//     feed: fill(t+1),                | math: intra(t) from the score tile, state update(t), stage O(t) into
+//           issue loads(t+2)          |       the X tile of block t (no longer read)
+//   ---- barrier ----
+// O(t-1) waits in the X tile of the set that fill(t+1) overwrites after the first barrier.
+// Both groups run their own loop; each executes exactly 1 + 2 * nblk barriers.
+constexpr int WS_THREADS = 512;
+constexpr int WS_XN = 0, WS_YN = BLK * LDN, WS_YT = 2 * BLK * LDN, WS_ZT = WS_YT + F * LDT;
+constexpr int WS_SET = WS_ZT + F * LDT;        // one block's tiles
+constexpr int WS_SC = 2 * WS_SET;              // the score tile
+constexpr int WS_LDS = WS_SC + BLK * LDSC;     // 144 384 B: one workgroup per CU
+
+template <class E, bool REV, bool TRANS>
+__device__ __forceinline__ void
+ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
+        const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out, const Geom &g,
+        int item, char *smem, const float *__restrict__ carry_in) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = w8 & 3;  // feed: score quadrant; math: column block
+  const int c = lane & 31, hh = lane >> 5;
+
+  const SegWork sw = seg_work(g, item);
+  const float sl = S[sw.bh % g.h] * LOG2E;
+  const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;
+  const int nblk = sw.nblk;
+  const int step = REV ? -1 : 1;
+  const int blk0 = REV ? nblk - 1 : 0;
+  const float blockdec = decay(sl, (float)BLK);
+
+  if (w8 < 4) {
+    // ================================ feed waves ================================
+    const int ftid = tid;  // 0..255
+    const LoaderRole xr = x_role(ftid), yr = yz_role(ftid);
+    const int chunk = ftid & 15, rowq = ftid >> 4;
+    const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + row0 * F);
+    const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * F);
+    const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * F);
+    u32x4 *Og = reinterpret_cast<u32x4 *>(Out + row0 * F);
+    constexpr int U = F / 4;  // 8-byte units per row
+    float kdec[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int b = 4 * yr.rowq + r;
+      kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
+    }
+    const int qI = w >> 1, qJ = w & 1;
+    const bool q_active = REV ? !(qI == 1 && qJ == 0) : !(qI == 0 && qJ == 1);
+    const uint32_t x_off = lane_offset(xr, xr.rowq, U), y_off = lane_offset(yr, 4 * yr.rowq, U);
+    const PieceMask all = {true, true};
+
+    // the block in flight, two 8-byte pieces per row (see LoaderRole)
+    u32x4 nx[4], ny[4], nz[4];
+    auto issue_loads = [&](int blk) __attribute__((always_inline)) {
+      const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * U * 8);
+      const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * U * 8);
+      const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * U * 8);
+#pragma unroll
+      for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(xblk, 16 * it * U * 8, x_off, all, true);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        ny[r] = load_row_pieces(yblk, r * U * 8, y_off, all, true);
+        nz[r] = load_row_pieces(zblk, r * U * 8, y_off, all, true);
+      }
+    };
+    // writes the block held in nx / ny / nz into a tile set: token-major X and Y, feature-major Y (scaled by the
+    // key decay) and Z
+    auto fill = [&](char *set) __attribute__((always_inline)) {
+#pragma unroll
+      for (int it = 0; it < 4; ++it)
+        *reinterpret_cast<u32x4 *>(set + WS_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        *reinterpret_cast<u32x4 *>(set + WS_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
+      store_transposed<E, true>(set + WS_YT, ny, yr, kdec);
+      store_transposed<E, false>(set + WS_ZT, nz, yr, kdec);
+    };
+    // the output tile staged in `set`'s X region -> global rows of block `blk`
+    auto store_out = [&](const char *set, int blk) __attribute__((always_inline)) {
+      const int64_t brow = (int64_t)blk * BLK;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int row = rowq + 16 * r4;
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(set + WS_XN + row * LDN + chunk * 16),
+                                    &Og[(brow + row) * (F / 8) + chunk]);
+      }
+    };
+    // this wave's quadrant of the transposed score tile: sc[4g+r] = y_b . x_a, b = 32qJ+8g+4hh+r, a = 32qI+c
+    auto score = [&](const char *set) __attribute__((always_inline)) {
+      if (!q_active) return;
+      floatx16 sc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+      const char *xa = set + WS_XN + (32 * qI + c) * LDN + hh * 16;
+      const char *ya = set + WS_YN + (32 * qJ + c) * LDN + hh * 16;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) sc = E::mfma(lds16(ya + ks * 32), lds16(xa + ks * 32), sc);
+      const int a = 32 * qI + c;
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        float m[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int b = 32 * qJ + 8 * gq + 4 * hh + r;
+          const int dist = REV ? b - a : a - b;
+          m[r] = dist >= 0 ? sc[4 * gq + r] * decay(sl, (float)dist) : 0.f;
+        }
+        u32x2 o;
+        o.x = E::pack(m[0], m[1]);
+        o.y = E::pack(m[2], m[3]);
+        *reinterpret_cast<u32x2 *>(smem + WS_SC + a * LDSC + (32 * qJ + 8 * gq + 4 * hh) * 2) = o;
+      }
+    };
+
+    issue_loads(blk0);
+    fill(smem);
+    if (nblk > 1) issue_loads(blk0 + step);
+    __syncthreads();  // barrier 0: block 0 visible
+    int blk = blk0;
+    for (int it = 0; it < nblk; ++it, blk += step) {
+      char *cur = smem + (it & 1) * WS_SET, *nxt = smem + ((it + 1) & 1) * WS_SET;
+      // the stores go first: by the time the fill below waits for its loads (loads and stores share one
+      // counter, so that wait drains both) they have long left
+      if (it > 0) store_out(nxt, blk - step);
+      score(cur);
+      __syncthreads();  // barrier 2 it + 1: score tile complete; X / Y of `cur` and the output staged in `nxt` no longer read
+      if (it + 1 < nblk) {
+        fill(nxt);
+        if (it + 2 < nblk) issue_loads(blk + 2 * step);
+      }
+      __syncthreads();  // barrier 2 it + 2: next block visible; output of this block staged
+    }
+    store_out(smem + ((nblk - 1) & 1) * WS_SET, blk0 + (nblk - 1) * step);
+    return;
+  }
+
+  // ================================== math waves ==================================
+  float qdec[2];
+#pragma unroll
+  for (int I = 0; I < 2; ++I) {
+    const int a = 32 * I + c;
+    qdec[I] = decay(sl, REV ? (float)(BLK - a) : (float)a);
+  }
+  // state entering the segment: st[T][4g+r] = St[32T+8g+4hh+r][32w+c]
+  floatx16 st[4];
+#pragma unroll
+  for (int T = 0; T < 4; ++T)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
+  if (states) {
+    // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
+    // the segment visited before it (the chunk's incoming state for the first one)
+    const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
+    bool have = true;
+    if (state_dies_in_segment(S[sw.bh % g.h], g)) {
+      const int nb = REV ? sw.seg + 1 : sw.seg - 1;
+      if (nb < 0 || nb >= g.n_seg) {
+        have = carry_in != nullptr;
+        src = carry_in + (int64_t)sw.bh * (F * F);
+      } else {
+        src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
+      }
+    }
+    if (have) {
+      typedef const __attribute__((address_space(1))) float *gmem_f32;
+      const uint32_t lane_off =
+          (uint32_t)(TRANS ? (32 * w + c) * F + 4 * hh : 4 * hh * F + 32 * w + c) * (uint32_t)sizeof(float);
+#pragma unroll
+      for (int T = 0; T < 4; ++T)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          const int band = 32 * T + 8 * gq;
+          const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : band * F)));
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            st[T][4 * gq + r] =
+                *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * F) * sizeof(float));
+        }
+    }
+  }
+  __syncthreads();  // barrier 0
+  for (int it = 0; it < nblk; ++it) {
+    char *cur = smem + (it & 1) * WS_SET;
+    // state term, transposed: acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
+    floatx16 acc[2];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc[0][r] = 0.f;
+      acc[1][r] = 0.f;
+    }
+    {
+      // all sixteen X fragments are requested before the first product (these waves have the registers for it)
+      const char *x0 = cur + WS_XN + c * LDN + hh * 16;
+      const char *x1 = x0 + 32 * LDN;
+      u32x4 xf[8][2];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        xf[ks][0] = lds16(x0 + ks * 32);
+        xf[ks][1] = lds16(x1 + ks * 32);
+      }
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int T = ks >> 1, u = ks & 1;
+        u32x4 a;
+        a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
+        a.y = E::pack(st[T][8 * u + 2], st[T][8 * u + 3]);
+        a.z = E::pack(st[T][8 * u + 4], st[T][8 * u + 5]);
+        a.w = E::pack(st[T][8 * u + 6], st[T][8 * u + 7]);
+        acc[0] = E::mfma(a, xf[ks][0], acc[0]);
+        acc[1] = E::mfma(a, xf[ks][1], acc[1]);
+      }
+    }
+#pragma unroll
+    for (int I = 0; I < 2; ++I)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[I][r] *= qdec[I];
+    __syncthreads();  // barrier 2 it + 1: score tile complete
+    {
+      u32x4 zf[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(cur + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
+      // the state has been consumed by the state term: decay it ahead of the update
+#pragma unroll
+      for (int T = 0; T < 4; ++T)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      // intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int I = 0; I < 2; ++I) {
+          const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
+          if (needed)
+            acc[I] = E::mfma(zf[u], lds16(smem + WS_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2), acc[I]);
+        }
+      // state update: St <- l^64 St + (scaled Y)^T Z
+      u32x4 yf[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int T = 0; T < 4; ++T) yf[u][T] = lds16(cur + WS_YT + tr_off(32 * T + c, 2 * u + hh));
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int T = 0; T < 4; ++T) st[T] = E::mfma(yf[u][T], zf[u], st[T]);
+    }
+    // stage the output tile (token-major) in the X region of this block
+#pragma unroll
+    for (int I = 0; I < 2; ++I)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        u32x2 o;
+        o.x = E::pack(acc[I][4 * gq + 0], acc[I][4 * gq + 1]);
+        o.y = E::pack(acc[I][4 * gq + 2], acc[I][4 * gq + 3]);
+        *reinterpret_cast<u32x2 *>(cur + WS_XN + (32 * I + c) * LDN + (32 * w + 8 * gq + 4 * hh) * 2) = o;
+      }
+    __syncthreads();  // barrier 2 it + 2
+  }
+}
+
+template <class E, bool REV, bool TRANS>
+__global__ void __launch_bounds__(WS_THREADS, 1)
+la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
+            const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
+            elem16_t *__restrict__ Out, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  ws_body<E, REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem, carry_in);
+}
+
+// la_bwd3 on the wave-specialised sweep (same triples, same placement)
+template <class E>
+__global__ void __launch_bounds__(WS_THREADS, 1)
+la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+           const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_states,
+           const float *__restrict__ dkv_states, const float *__restrict__ kv_in, const float *__restrict__ dkv_in,
+           elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  const int n_items = g.b * g.h * g.n_seg;
+  const int grp = blockIdx.x / 24, r = blockIdx.x - grp * 24;
+  const int role = r >> 3;
+  const int item = n_items - 1 - (grp * 8 + (r & 7));
+  if (item < 0) return;
+  if (role == 0)
+    ws_body<E, false, true>(DO, V, K, S, kv_states, DQ, g, item, smem, kv_in);
+  else if (role == 1)
+    ws_body<E, true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem, dkv_in);
+  else
+    ws_body<E, true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem, dkv_in);
+}
+
+// ------------------------------------------------------------------------------
 // A segment's own state:  causal  sum_b l^(L-b) y_b^T z_b ;  anti-causal  sum_b l^b y_b^T z_b
 // (b from the segment start, L its length), written token-free as 128 x 128 fp32.  Y rows hold
 // g.d features and Z rows g.e (M_NARROW; 128 otherwise).
@@ -801,7 +1104,7 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
 // Blocks whose every token carries a weight below 2^-SKIP_LOG2 are neither read nor multiplied:
 // with slope s a token that lies x tokens from the segment's far end weighs exp(-s x), so a
 // fast-decaying head only needs the last (causal) or first (anti-causal) SKIP_LOG2 ln2 / s tokens
-// of each segment.  What is dropped is below 2^-64 of a full-weight term, far under the fp32
+// of each segment.  What is dropped is below 2^-24 of a full-weight term, i.e. under the fp32
 // rounding (2^-24) of the sum it would be added to.  s = 0 skips nothing.
 //
 // That leaves the workgroups unevenly loaded -- those of slow-decaying heads still read whole
@@ -989,6 +1292,33 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
+template <class E, bool REV, bool TRANS>
+int launch_apply_ws(const void *x, const void *y, const void *z, const float *s, const float *states,
+                    const float *carry_in, void *out, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_apply_ws<E, REV, TRANS>>(WS_LDS);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_APPLY, st);
+  la_apply_ws<E, REV, TRANS><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
+                                                                 (const elem16_t *)z, s, states, carry_in,
+                                                                 (elem16_t *)out, g);
+  return (int)hipGetLastError();
+}
+
+template <class E>
+int launch_bwd3_ws(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
+                   hipStream_t st) {
+  int rc = grant_lds<la_bwd3_ws<E>>(WS_LDS);
+  if (rc) return rc;
+  const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
+  const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
+  ProfScope prof(KC_BWD3, st);
+  la_bwd3_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k, (const elem16_t *)a.v,
+                                                    (const elem16_t *)a.d_o, a.s, kv_states, dkv_states, a.kv_in,
+                                                    a.dkv_in, (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
+  return (int)hipGetLastError();
+}
+
 // skip_seg: the segment whose own state nothing reads (-1: none); its workgroups leave at once
 template <class E, bool REV, int MODE>
 int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
@@ -1051,6 +1381,9 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
+  if (MODE == M_ALIGNED && g.ws)
+    return launch_apply_ws<E, false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.kv_in, a.o, g,
+                                            st);
   return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
                                                           a.kv_in, nullptr, a.o, g, st);
 }
@@ -1081,6 +1414,7 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
+  if (MODE == M_ALIGNED && g.ws) return launch_bwd3_ws<E>(a, kv_states, dkv_states, g, st);
   return launch_bwd3<E, MODE, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
 }
 
