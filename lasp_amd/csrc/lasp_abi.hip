@@ -2,7 +2,6 @@
 // the kernel families.  Declarations and the tensor contract: include/lasp_hip.h.
 #include <stdarg.h>
 #include <stdio.h>
-#include <stdlib.h>
 
 #include <atomic>
 
@@ -139,7 +138,10 @@ constexpr int kFusedMaxWalk = 8;  // blocks
 // (each workgroup re-runs the scan's recurrence over at most kCombineMaxSeg - 1 states of 64 KiB)
 // and the scan launch is dropped; with one segment the pre-pass goes too.  Measured at b*h = 24,
 // n = 2048: 4 segments 84 against 88 us forward + backward, 8 segments 137 against 100 us (the
-// gathers grow with the square of the segment count), hence the limit.
+// gathers grow with the square of the segment count), hence the limit.  The wave-specialised sweeps gather only as
+// far back as a head's decay reaches and while their other waves fetch the first block; at 7 segments that still
+// costs what the scan launch saves (b*h = 24, n = 2048: 67 against 69 us per chunk in kernels, 691 against 677 us
+// for the 8-chunk chain replayed from a graph), so the limit stays.
 constexpr int64_t kCombineMaxSeg = 4;
 bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg_len, int64_t n_seg) {
   if (seg_len_arg != 0 || !mfma_eligible(d, e, dtype) || n > kFusedMaxTokens) return false;
@@ -174,10 +176,8 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
                 n_seg <= kCombineMaxSeg) ? 1 : 0;
   // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
   g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg >= 2) ? 1 : 0;
-  {
-    const char *ev = getenv("LASP_WS");  // experiment switch
-    g->ws = ((!ev || atoi(ev) != 0) && mfma_eligible(d, e, dtype) && !g->fused && !g->combine) ? 1 : 0;
-  }
+  // full-width 16-bit heads on a chunk of whole blocks take the wave-specialised sweeps
+  g->ws = (mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature && n % kSegQuantum == 0 && !g->fused) ? 1 : 0;
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;

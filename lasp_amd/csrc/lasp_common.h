@@ -60,7 +60,7 @@ struct Geom {
   int fused;    // the chunk is served by the single-launch kernels, which use no workspace
   int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
   int bypass;   // the scan leaves out heads whose state dies within one segment (see state_dies_in_segment)
-  int ws;       // aligned 16-bit chunks on the scan path run the wave-specialised sweeps (la_apply_ws, la_bwd3_ws)
+  int ws;       // d = e = 128, 16-bit, n a multiple of 64, not fused: the sweeps run wave-specialised (la_apply_ws, la_bwd3_ws)
 };
 
 // Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels.  A state is an fp32 sum

@@ -817,11 +817,12 @@ constexpr int WS_SET = WS_ZT + F * LDT;        // one block's tiles
 constexpr int WS_SC = 2 * WS_SET;              // the score tile
 constexpr int WS_LDS = WS_SC + BLK * LDSC;     // 144 384 B: one workgroup per CU
 
-template <class E, bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS, int SRC>
 __device__ __forceinline__ void
 ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out, const Geom &g,
-        int item, char *smem, const float *__restrict__ carry_in) {
+        int item, char *smem, const float *__restrict__ carry_in, float *__restrict__ carry_out = nullptr) {
+  static_assert(SRC == SRC_SCANNED || SRC == SRC_COMBINE, "the wave-specialised sweep takes its state from the workspace");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -955,35 +956,63 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
   for (int T = 0; T < 4; ++T)
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
-  if (states) {
-    // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
-    // the segment visited before it (the chunk's incoming state for the first one)
-    const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
-    bool have = true;
-    if (state_dies_in_segment(S[sw.bh % g.h], g)) {
-      const int nb = REV ? sw.seg + 1 : sw.seg - 1;
-      if (nb < 0 || nb >= g.n_seg) {
-        have = carry_in != nullptr;
-        src = carry_in + (int64_t)sw.bh * (F * F);
-      } else {
-        src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
+  // st <- f * st + M, M being the 128 x 128 fp32 matrix at `src` (read transposed by the transposed roles)
+  auto add_state = [&](const float *src, float f) __attribute__((always_inline)) {
+    typedef const __attribute__((address_space(1))) float *gmem_f32;
+    const uint32_t lane_off =
+        (uint32_t)(TRANS ? (32 * w + c) * F + 4 * hh : 4 * hh * F + 32 * w + c) * (uint32_t)sizeof(float);
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        const int band = 32 * T + 8 * gq;
+        const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : band * F)));
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          st[T][4 * gq + r] = fmaf(
+              f, st[T][4 * gq + r],
+              *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * F) * sizeof(float)));
       }
-    }
-    if (have) {
-      typedef const __attribute__((address_space(1))) float *gmem_f32;
-      const uint32_t lane_off =
-          (uint32_t)(TRANS ? (32 * w + c) * F + 4 * hh : 4 * hh * F + 32 * w + c) * (uint32_t)sizeof(float);
-#pragma unroll
-      for (int T = 0; T < 4; ++T)
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          const int band = 32 * T + 8 * gq;
-          const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : band * F)));
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            st[T][4 * gq + r] =
-                *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * F) * sizeof(float));
+  };
+  if (SRC == SRC_SCANNED) {
+    if (states) {
+      // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
+      // the segment visited before it (the chunk's incoming state for the first one)
+      const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
+      bool have = true;
+      if (state_dies_in_segment(S[sw.bh % g.h], g)) {
+        const int nb = REV ? sw.seg + 1 : sw.seg - 1;
+        if (nb < 0 || nb >= g.n_seg) {
+          have = carry_in != nullptr;
+          src = carry_in + (int64_t)sw.bh * (F * F);
+        } else {
+          src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
         }
+      }
+      if (have) add_state(src, 0.f);
+    }
+  } else {
+    // `states` holds the segments' OWN states.  The scan's recurrence, St <- l^len_j St + own_j over the
+    // segments visited before this one, is run here -- over as many of them as the head's decay reaches:
+    // an own state further back arrives weighted below 2^-SKIP_LOG2 (everything between it and this
+    // segment is a full-length segment) and is left out, and so is the chunk's incoming state unless the
+    // walk starts at the chunk's end.  These waves have the time: the feed waves are fetching block 0.
+    const int n_before = REV ? g.n_seg - 1 - sw.seg : sw.seg;
+    int first = 0;
+    if (sl > 0.f) {
+      const float segs = SKIP_LOG2 / (sl * (float)g.seg_len);  // full segments over which a weight falls to 2^-SKIP_LOG2
+      if (segs < (float)n_before) first = n_before - ((int)segs + 1);
+    }
+    first = __builtin_amdgcn_readfirstlane(first);
+    if (first == 0 && carry_in) add_state(carry_in + (int64_t)sw.bh * (F * F), 0.f);
+    if (states) {
+      const float *base = states + (int64_t)sw.bh * g.n_seg * (F * F);
+      const float full = decay(sl, (float)g.seg_len);
+      const float last = decay(sl, (float)(g.n - (int64_t)(g.n_seg - 1) * g.seg_len));
+      for (int i = first; i < n_before; ++i) {
+        const int j = REV ? g.n_seg - 1 - i : i;
+        add_state(base + (int64_t)j * (F * F), j == g.n_seg - 1 ? last : full);
+      }
     }
   }
   __syncthreads();  // barrier 0
@@ -1064,24 +1093,35 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       }
     __syncthreads();  // barrier 2 it + 2
   }
+  // the segment visited last leaves the chunk's outgoing state
+  if (SRC == SRC_COMBINE && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
+    float *cp = carry_out + (int64_t)sw.bh * (F * F);
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) cp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
+  }
 }
 
-template <class E, bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS, int SRC>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
             const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
-            elem16_t *__restrict__ Out, Geom g) {
+            float *__restrict__ carry_out, elem16_t *__restrict__ Out, Geom g) {
   extern __shared__ __align__(16) char smem[];
-  ws_body<E, REV, TRANS>(X, Y, Z, S, states, Out, g, (int)blockIdx.x, smem, carry_in);
+  // SRC_COMBINE: later segments have more states to gather first, so they are started first
+  const int item = SRC == SRC_COMBINE ? g.b * g.h * g.n_seg - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  ws_body<E, REV, TRANS, SRC>(X, Y, Z, S, states, Out, g, item, smem, carry_in, carry_out);
 }
 
 // la_bwd3 on the wave-specialised sweep (same triples, same placement)
-template <class E>
+template <class E, int SRC>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
            const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_states,
            const float *__restrict__ dkv_states, const float *__restrict__ kv_in, const float *__restrict__ dkv_in,
-           elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
+           float *__restrict__ dkv_out, elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK,
+           elem16_t *__restrict__ DV, Geom g) {
   extern __shared__ __align__(16) char smem[];
   const int n_items = g.b * g.h * g.n_seg;
   const int grp = blockIdx.x / 24, r = blockIdx.x - grp * 24;
@@ -1089,11 +1129,11 @@ la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    ws_body<E, false, true>(DO, V, K, S, kv_states, DQ, g, item, smem, kv_in);
+    ws_body<E, false, true, SRC>(DO, V, K, S, kv_states, DQ, g, item, smem, kv_in);
   else if (role == 1)
-    ws_body<E, true, false>(K, Q, DO, S, dkv_states, DV, g, item, smem, dkv_in);
+    ws_body<E, true, false, SRC>(K, Q, DO, S, dkv_states, DV, g, item, smem, dkv_in, dkv_out);
   else
-    ws_body<E, true, true>(V, DO, Q, S, dkv_states, DK, g, item, smem, dkv_in);
+    ws_body<E, true, true, SRC>(V, DO, Q, S, dkv_states, DK, g, item, smem, dkv_in);
 }
 
 // ------------------------------------------------------------------------------
@@ -1292,30 +1332,31 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
-template <class E, bool REV, bool TRANS>
+template <class E, bool REV, bool TRANS, int SRC>
 int launch_apply_ws(const void *x, const void *y, const void *z, const float *s, const float *states,
-                    const float *carry_in, void *out, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_apply_ws<E, REV, TRANS>>(WS_LDS);
+                    const float *carry_in, float *carry_out, void *out, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_apply_ws<E, REV, TRANS, SRC>>(WS_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply_ws<E, REV, TRANS><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
-                                                                 (const elem16_t *)z, s, states, carry_in,
-                                                                 (elem16_t *)out, g);
+  la_apply_ws<E, REV, TRANS, SRC><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
+                                                                      (const elem16_t *)z, s, states, carry_in,
+                                                                      carry_out, (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
-template <class E>
+template <class E, int SRC>
 int launch_bwd3_ws(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                    hipStream_t st) {
-  int rc = grant_lds<la_bwd3_ws<E>>(WS_LDS);
+  int rc = grant_lds<la_bwd3_ws<E, SRC>>(WS_LDS);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k, (const elem16_t *)a.v,
-                                                    (const elem16_t *)a.d_o, a.s, kv_states, dkv_states, a.kv_in,
-                                                    a.dkv_in, (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
+  la_bwd3_ws<E, SRC><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
+                                                         kv_states, dkv_states, a.kv_in, a.dkv_in, a.dkv_out,
+                                                         (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
   return (int)hipGetLastError();
 }
 
@@ -1373,6 +1414,9 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if (g.n_seg > 1 &&
         (rc = launch_state_skipping<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, g.n_seg - 1, st)))
       return rc;
+    if (MODE == M_ALIGNED && g.ws)
+      return launch_apply_ws<E, false, false, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
+                                                           a.kv_in, a.kv_out, a.o, g, st);
     return launch_apply<E, false, false, MODE, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
                                                             a.kv_in, a.kv_out, a.o, g, st);
   }
@@ -1382,8 +1426,8 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
   }
   if (MODE == M_ALIGNED && g.ws)
-    return launch_apply_ws<E, false, false>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr, a.kv_in, a.o, g,
-                                            st);
+    return launch_apply_ws<E, false, false, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
+                                                         a.kv_in, nullptr, a.o, g, st);
   return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
                                                           a.kv_in, nullptr, a.o, g, st);
 }
@@ -1399,6 +1443,8 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
       kv_states = a.ws_kv;
     }
     if (g.n_seg > 1 && (rc = launch_state_skipping<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, 0, st))) return rc;
+    if (MODE == M_ALIGNED && g.ws)
+      return launch_bwd3_ws<E, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
     return launch_bwd3<E, MODE, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g,
                                              st);
   }
@@ -1414,7 +1460,7 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  if (MODE == M_ALIGNED && g.ws) return launch_bwd3_ws<E>(a, kv_states, dkv_states, g, st);
+  if (MODE == M_ALIGNED && g.ws) return launch_bwd3_ws<E, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
   return launch_bwd3<E, MODE, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
 }
 
