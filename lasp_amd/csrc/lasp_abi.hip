@@ -61,6 +61,7 @@ constexpr int kMinSeg = 256;
 constexpr int kPreferredSeg = 1024;     // preferred lower bound while kMinGroups workgroups remain
 constexpr int64_t kMinGroups = 256;     // one workgroup per CU
 constexpr int64_t kMaxSeg = 1 << 24;    // offsets inside a segment stay within 32 bits
+constexpr int kPreMaxSeg = 2048;        // longest segment the pre-pass walks in one workgroup (see make_geom)
 
 int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
   if (dtype != LASP_DTYPE_F32 && dtype != LASP_DTYPE_BF16 && dtype != LASP_DTYPE_F16) {
@@ -164,20 +165,44 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     set_error("too many segments (%lld) for seg_len=%d", (long long)n_seg, seg_len);
     return LASP_E_SEGMENT;
   }
+  const bool ws = mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature && n % kSegQuantum == 0 &&
+                  !fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg);
+  if (ws && seg_len_arg == 0 && n_seg > kCombineMaxSeg) {
+    // The wave-specialised sweeps hold a CU each, so the default plan aims at one round of 256 workgroups in the
+    // forward sweep rather than two per CU: longer segments mean fewer states to load and carry (b*h = 16,
+    // n = 65536: 4096-token segments, sweeps 193 + 496 us against 201 + 513 with 2048; b*h = 32, n = 16384:
+    // 2048 against 1024, 97 + 248 against 102 + 256).
+    while ((int64_t)b * h * ((n + 2 * seg_len - 1) / (2 * seg_len)) >= kMinGroups &&
+           (n + 2 * seg_len - 1) / (2 * seg_len) > kCombineMaxSeg)
+      seg_len *= 2;
+  }
+  const int64_t n_seg_final = (n + seg_len - 1) / seg_len;
   g->b = b;
   g->h = h;
   g->n = n;
   g->d = d;
   g->e = e;
   g->seg_len = seg_len;
-  g->n_seg = (int)n_seg;
-  g->fused = fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg) ? 1 : 0;
+  g->n_seg = (int)n_seg_final;
+  g->fused = fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg_final) ? 1 : 0;
   g->combine = (!g->fused && mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature &&
-                n_seg <= kCombineMaxSeg) ? 1 : 0;
+                n_seg_final <= kCombineMaxSeg) ? 1 : 0;
   // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
-  g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg >= 2) ? 1 : 0;
+  g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg_final >= 2) ? 1 : 0;
   // full-width 16-bit heads on a chunk of whole blocks take the wave-specialised sweeps
   g->ws = (mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature && n % kSegQuantum == 0 && !g->fused) ? 1 : 0;
+  // The pre-pass walks a segment serially, and its slow-decay heads walk all of it: beyond 2048 tokens that
+  // walk outlasts everything else in the launch (b*h = 16, n = 65536: 71 us at 4096 tokens against 51 at
+  // 2048; at 1024 the extra states cost more again, 62 us and a longer scan).  Long sweep segments are therefore cut in halves (quarters, ...) for the pre-pass and the scan, and
+  // a sweep takes the state that enters its first piece.  A pure function of the shape and seg_len, so that a
+  // backward call given the forward's seg_len finds the states where the forward left them.
+  g->pre_len = seg_len;
+  if (g->ws && !g->combine) {
+    int pre = seg_len;
+    while (pre > kPreMaxSeg && pre % (2 * kSegQuantum) == 0) pre /= 2;
+    if (pre <= kPreMaxSeg) g->pre_len = pre;
+  }
+  g->pre_n = (int)((n + g->pre_len - 1) / g->pre_len);
   const bool padded_states = mfma_eligible(d, e, dtype) || mfma_f32_eligible(d, e, dtype);
   g->sd = padded_states ? kMaxFeature : d;
   g->se = padded_states ? kMaxFeature : e;
@@ -283,7 +308,7 @@ int static_scratch(float **out) {
 }
 
 size_t state_bytes_of(const Geom &g) {
-  return sizeof(float) * (size_t)g.b * g.h * g.n_seg * g.sd * g.se;
+  return sizeof(float) * (size_t)g.b * g.h * g.pre_n * g.sd * g.se;
 }
 
 }  // namespace

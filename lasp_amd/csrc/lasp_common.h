@@ -60,6 +60,9 @@ struct Geom {
   int fused;    // the chunk is served by the single-launch kernels, which use no workspace
   int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
   int bypass;   // the scan leaves out heads whose state dies within one segment (see state_dies_in_segment)
+  int pre_len;  // tokens per segment of the pre-pass and the scan: seg_len, or seg_len / 2^k where long sweep
+                // segments are cut finer for the pre-pass (wave-specialised scan path only)
+  int pre_n;    // ceil(n / pre_len): states per (b, h) in the workspace
   int ws;       // d = e = 128, 16-bit, n a multiple of 64, not fused: the sweeps run wave-specialised (la_apply_ws, la_bwd3_ws)
 };
 
@@ -70,14 +73,14 @@ struct Geom {
 constexpr float kSkipLog2 = 24.f;
 constexpr float kLog2e = 1.4426950408889634f;
 
-// With g.bypass set, a head whose decay over the chunk's shortest segment (the last one) is below
+// With g.bypass set, a head whose decay over the shortest segment of the pre-pass (the last one) is below
 // 2^-kSkipLog2 takes no part in the scan: whatever enters a segment has faded to nothing at its far
 // end, so the state entering segment j is the OWN state of the segment before it (after it, going
 // backwards) and, for the first segment visited, the chunk's incoming state.  The scan kernel
 // leaves those heads' own states in place and only forms their outgoing carry; the sweeps read the
 // neighbour's own state.  Both sides must take the same decision, hence this one function.
 __device__ __forceinline__ bool state_dies_in_segment(float slope, const Geom &g) {
-  const int64_t last_len = g.n - (int64_t)(g.n_seg - 1) * g.seg_len;
+  const int64_t last_len = g.n - (int64_t)(g.pre_n - 1) * g.pre_len;  // segments of the pre-pass and the scan
   return g.bypass != 0 && slope * kLog2e * (float)last_len > kSkipLog2;
 }
 

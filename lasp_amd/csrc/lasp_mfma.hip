@@ -978,15 +978,20 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     if (states) {
       // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
       // the segment visited before it (the chunk's incoming state for the first one)
-      const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
+      // The workspace holds one state per segment of the pre-pass, of which this sweep segment spans
+      // `sub` (a power of two; 1 unless the plan cut long segments finer for the pre-pass): the state that
+      // enters it is the one entering its first piece in sweep order.
+      const int sub = g.seg_len / g.pre_len;
+      const int piece = REV ? min(sw.seg * sub + sub, g.pre_n) - 1 : sw.seg * sub;
+      const float *src = states + ((int64_t)sw.bh * g.pre_n + piece) * (F * F);
       bool have = true;
       if (state_dies_in_segment(S[sw.bh % g.h], g)) {
-        const int nb = REV ? sw.seg + 1 : sw.seg - 1;
-        if (nb < 0 || nb >= g.n_seg) {
+        const int nb = REV ? piece + 1 : piece - 1;
+        if (nb < 0 || nb >= g.pre_n) {
           have = carry_in != nullptr;
           src = carry_in + (int64_t)sw.bh * (F * F);
         } else {
-          src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
+          src = states + ((int64_t)sw.bh * g.pre_n + nb) * (F * F);
         }
       }
       if (have) add_state(src, 0.f);
@@ -1404,6 +1409,15 @@ int launch_fused_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// The geometry the pre-pass and the scan work on: the chunk cut into g.pre_n segments of g.pre_len tokens
+// (the sweeps' own segments unless the plan cut those finer for the pre-pass).
+Geom pre_pass_geom(const Geom &g) {
+  Geom gp = g;
+  gp.seg_len = g.pre_len;
+  gp.n_seg = g.pre_n;
+  return gp;
+}
+
 template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   if (g.fused) return launch_fused_fwd<E, MODE>(a, g, st);
@@ -1421,9 +1435,10 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
                                                             a.kv_in, a.kv_out, a.o, g, st);
   }
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
+  const Geom gp = pre_pass_geom(g);
   if (need_states) {
-    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, a.kv_out != nullptr, st))) return rc;
-    if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, g, 0, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, gp, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, gp, 0, st))) return rc;
   }
   if (MODE == M_ALIGNED && g.ws)
     return launch_apply_ws<E, false, false, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
@@ -1448,16 +1463,17 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     return launch_bwd3<E, MODE, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g,
                                              st);
   }
+  const Geom gp = pre_pass_geom(g);
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, g, false, st))) return rc;
-    if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, g, 0, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, gp, false, st))) return rc;
+    if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, gp, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, a.dkv_out != nullptr, st))) return rc;
-    if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, g, 1, st))) return rc;
+    if ((rc = launch_state<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, gp, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, gp, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
   if (MODE == M_ALIGNED && g.ws) return launch_bwd3_ws<E, SRC_SCANNED>(a, kv_states, dkv_states, g, st);

@@ -46,8 +46,16 @@ def test_library_exports_every_declared_symbol(lib):
 def test_plan_defaults_and_overrides(lib):
     from lasp_amd import _abi
 
-    # headline shape: 16 (b,h) pairs -> 32 segments of 2048 tokens = 512 workgroups
-    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16) == (2048, 32, 16 * 32 * 128 * 128 * 4)
+    # headline shape: 16 (b,h) pairs -> 16 sweep segments of 4096 tokens = 256 workgroups of the wave-specialised
+    # sweeps, one per CU; the pre-pass and the scan work on halves of them, so the workspace holds 32 states per (b,h)
+    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16) == (4096, 16, 16 * 32 * 128 * 128 * 4)
+    # an explicit seg_len gets the same treatment (the backward is handed the forward's seg_len)
+    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 4096) == (4096, 16, 16 * 32 * 128 * 128 * 4)
+    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 2048) == (2048, 32, 16 * 32 * 128 * 128 * 4)
+    assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 8192) == (8192, 8, 16 * 32 * 128 * 128 * 4)
+    # ragged or narrow rows stay on the two-per-CU kernels and their plan
+    assert _abi.plan(1, 16, 65536 + 8, 128, 128, torch.bfloat16)[:2] == (2304, 29)
+    assert _abi.plan(1, 16, 65536, 128, 64, torch.bfloat16) == (2048, 32, 16 * 32 * 128 * 128 * 4)
     # short chunk: 256 tokens per segment at least ...
     assert _abi.plan(1, 16, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
     # ... or 192 where even the backward's 3 workgroups per segment leave the chip under-filled

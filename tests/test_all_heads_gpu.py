@@ -3,8 +3,8 @@
 The pre-pass skips blocks whose weights lie below 2^-24, the scan leaves out heads whose state dies
 within one segment, and both only take effect on long segments.  Here every (batch, head) slice of every
 output is held to the oracle (fp32 block recurrence on the same rounded inputs) under the 2e-2 bound, on
-the pre-pass / scan / sweep path (6 segments of 2048 tokens and the planned segment length) and on the
-scan-less path (4 segments of 2048), with incoming KV and dKV states, with the forward's segment states
+the pre-pass / scan / sweep path (6 segments of 2048 tokens, the planned segment length, and 6 sweep segments
+of 4096 tokens over a pre-pass on halves of them) and on the scan-less path (4 segments of 2048), with incoming KV and dKV states, with the forward's segment states
 kept for the backward and with the backward recomputing them.  Slope sets: the benchmark's schedule,
 and one built around the shortcuts' thresholds (no decay, the pre-pass reaching exactly one block, the
 scan's cut-off at the segment length just met and just missed)."""
@@ -56,14 +56,15 @@ def _run(inp, s, seg_len, cache):
 
 
 @pytest.mark.parametrize("slope_set", ["baseline", "thresholds"])
-@pytest.mark.parametrize("n,seg_len", [(12288, 2048), (12288, 0), (8192, 2048), (8192, 0)],
-                         ids=["scan_6x2048", "scan_planned", "combine_4x2048", "planned_8192"])
+@pytest.mark.parametrize("n,seg_len", [(12288, 2048), (12288, 0), (8192, 2048), (8192, 0), (24576, 4096)],
+                         ids=["scan_6x2048", "scan_planned", "combine_4x2048", "planned_8192", "scan_6x4096_prepass_2048"])
 def test_every_head_with_states(gpu_device, slope_set, n, seg_len):
     from lasp_amd import _abi
 
     dev = gpu_device
     planned = _abi.plan(1, H, n, D, D, torch.bfloat16, seg_len)[0]
-    s = O.slopes_baseline(H) if slope_set == "baseline" else _threshold_slopes(planned)
+    # the scan's cut-off works on the pre-pass's segments, which are at most 2048 tokens long
+    s = O.slopes_baseline(H) if slope_set == "baseline" else _threshold_slopes(min(planned, 2048))
     inp = _inputs(n, dev, seed=500 + n // 1024 + seg_len)
     cpu = {k_: t.cpu() for k_, t in inp.items()}
     ref = O.ref_chunked(cpu["q"], cpu["k"], cpu["v"], s, cpu["do"], cpu["kv"], cpu["dkv"], dtype=torch.float32)
