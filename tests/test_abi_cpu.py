@@ -150,6 +150,42 @@ def test_in_place_state_update_rules(lib):
     assert bwd(512, 64) == -7
 
 
+def test_documented_launch_shims_run_as_written(lib, monkeypatch):
+    """The reference-side binding shown in INTEGRATION.md (its python blocks, executed as they stand) must get
+    past the library's argument checks on the reference's own per-rank test shape, n = 512, where the kernels
+    cannot update a state in place: with host tensors the call that stops it is the device check, not
+    LASP_E_ALIAS."""
+    import contextlib
+    import types
+
+    from lasp_amd import _abi
+
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = [b for b in re.findall(r"```python\n(.*?)```", text, flags=re.S) if "_lib" in b or "_plan(" in b]
+    assert len(blocks) == 3, "expected the binding, lasp_forward and lasp_backward blocks"
+    code = "\n".join(blocks).replace("/path/to/lasp_amd/liblasp_hip.so", _abi.lib_path())
+    monkeypatch.setattr(torch.cuda, "device", lambda idx: contextlib.nullcontext())
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda *a: types.SimpleNamespace(cuda_stream=0))
+    ns = {}
+    exec(compile(code, "INTEGRATION.md", "exec"), ns)
+
+    b, h, n, d = 2, 12, 512, 128
+    assert not _abi.inplace_ok(b, h, n, d, d, torch.bfloat16, ns["_plan"](torch.empty(b, h, n, d, dtype=torch.bfloat16),
+                                                                          torch.empty(b, h, n, d))[0], False)
+    q, k, v, do = [torch.zeros(b, h, n, d, dtype=torch.bfloat16) for _ in range(4)]
+    s = torch.ones(h)
+    KV, DKV = torch.zeros(b, h, d, d), torch.zeros(b, h, d, d)
+    with pytest.raises(RuntimeError, match="not a device pointer|current device"):
+        ns["lasp_forward"](q, k, v, s, KV)
+    with pytest.raises(RuntimeError, match="not a device pointer|current device"):
+        ns["lasp_backward"](q, k, v, s, do, KV.clone(), DKV)
+    # the same calls with the state buffer on both sides are what the library refuses
+    seg, _ = ns["_plan"](q, v)
+    rc = ns["_lib"].lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), KV.data_ptr(), KV.data_ptr(),
+                                   q.data_ptr(), k.data_ptr(), b, h, n, d, d, 1, seg, None)
+    assert rc == -8
+
+
 def test_alignment_and_device_errors_need_no_gpu(lib):
     """A misaligned tensor or state pointer is LASP_E_ALIGN; a pointer HIP does not know as memory of
     the current device is LASP_E_DEVICE.  Both are reported before anything is launched."""
