@@ -822,7 +822,6 @@ __device__ __forceinline__ void
 ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out, const Geom &g,
         int item, char *smem, const float *__restrict__ carry_in, float *__restrict__ carry_out = nullptr) {
-  static_assert(SRC == SRC_SCANNED || SRC == SRC_COMBINE, "the wave-specialised sweep takes its state from the workspace");
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -836,6 +835,28 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
   const int step = REV ? -1 : 1;
   const int blk0 = REV ? nblk - 1 : 0;
   const float blockdec = decay(sl, (float)BLK);
+
+  // SRC_WALK: the state entering the segment is rebuilt by walking `runup` blocks outside it first (before it,
+  // or after it going backwards), as far as the head's decay reaches, from the chunk's incoming state if the
+  // walk gets to the chunk's end, else from zero.  Blocks are numbered relative to the segment; walk and sweep
+  // form one run of runup + nblk blocks, first_blk, first_blk + step, ..., of which the first `runup` only
+  // update the state (one barrier each, both groups).
+  int runup = 0;
+  bool take_carry = false;
+  if (SRC == SRC_WALK) {
+    const int total_blk = (int)(g.n / BLK);
+    const int seg_blk0 = (int)(sw.tok0 / BLK);
+    const int avail = REV ? total_blk - (seg_blk0 + nblk) : seg_blk0;
+    int reach = avail;
+    if (sl > 0.f) {
+      const float x = SKIP_LOG2 / (sl * (float)BLK);  // blocks over which a weight falls to 2^-SKIP_LOG2
+      if (x < (float)avail) reach = (int)x + 1;
+    }
+    runup = __builtin_amdgcn_readfirstlane(min(reach, avail));
+    take_carry = carry_in != nullptr && runup == avail;
+  }
+  const int first_blk = blk0 - runup * step;
+  const int run = runup + nblk;  // blocks in the whole run
 
   if (w8 < 4) {
     // ================================ feed waves ================================
@@ -860,12 +881,16 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
 
     // the block in flight, two 8-byte pieces per row (see LoaderRole)
     u32x4 nx[4], ny[4], nz[4];
-    auto issue_loads = [&](int blk) __attribute__((always_inline)) {
+    // k: position in the run; walk blocks (k < runup) need no X tile
+    auto issue_loads = [&](int k) __attribute__((always_inline)) {
+      const int blk = first_blk + k * step;
       const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * U * 8);
       const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * U * 8);
       const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * U * 8);
+      if (SRC != SRC_WALK || k >= runup) {
 #pragma unroll
-      for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(xblk, 16 * it * U * 8, x_off, all, true);
+        for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(xblk, 16 * it * U * 8, x_off, all, true);
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         ny[r] = load_row_pieces(yblk, r * U * 8, y_off, all, true);
@@ -874,13 +899,15 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     };
     // writes the block held in nx / ny / nz into a tile set: token-major X and Y, feature-major Y (scaled by the
     // key decay) and Z
-    auto fill = [&](char *set) __attribute__((always_inline)) {
+    auto fill = [&](char *set, int k) __attribute__((always_inline)) {
+      if (SRC != SRC_WALK || k >= runup) {  // a walk block is only multiplied into the state
 #pragma unroll
-      for (int it = 0; it < 4; ++it)
-        *reinterpret_cast<u32x4 *>(set + WS_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
+        for (int it = 0; it < 4; ++it)
+          *reinterpret_cast<u32x4 *>(set + WS_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        *reinterpret_cast<u32x4 *>(set + WS_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
+        for (int r = 0; r < 4; ++r)
+          *reinterpret_cast<u32x4 *>(set + WS_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
+      }
       store_transposed<E, true>(set + WS_YT, ny, yr, kdec);
       store_transposed<E, false>(set + WS_ZT, nz, yr, kdec);
     };
@@ -921,25 +948,30 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       }
     };
 
-    issue_loads(blk0);
-    fill(smem);
-    if (nblk > 1) issue_loads(blk0 + step);
-    __syncthreads();  // barrier 0: block 0 visible
-    int blk = blk0;
-    for (int it = 0; it < nblk; ++it, blk += step) {
-      char *cur = smem + (it & 1) * WS_SET, *nxt = smem + ((it + 1) & 1) * WS_SET;
+    issue_loads(0);
+    fill(smem, 0);
+    if (run > 1) issue_loads(1);
+    __syncthreads();  // barrier 0: block 0 of the run visible
+    int k = 0;
+    for (; k < runup; ++k) {  // walk: the math waves multiply block k into the state meanwhile
+      fill(smem + ((k + 1) & 1) * WS_SET, k + 1);  // k + 1 < run: a sweep block follows the walk
+      if (k + 2 < run) issue_loads(k + 2);
+      __syncthreads();  // walk barrier k
+    }
+    for (; k < run; ++k) {
+      char *cur = smem + (k & 1) * WS_SET, *nxt = smem + ((k + 1) & 1) * WS_SET;
       // the stores go first: by the time the fill below waits for its loads (loads and stores share one
       // counter, so that wait drains both) they have long left
-      if (it > 0) store_out(nxt, blk - step);
+      if (k > runup) store_out(nxt, first_blk + (k - 1) * step);
       score(cur);
-      __syncthreads();  // barrier 2 it + 1: score tile complete; X / Y of `cur` and the output staged in `nxt` no longer read
-      if (it + 1 < nblk) {
-        fill(nxt);
-        if (it + 2 < nblk) issue_loads(blk + 2 * step);
+      __syncthreads();  // first barrier of a sweep block: score tile complete; X / Y of `cur` and the output staged in `nxt` no longer read
+      if (k + 1 < run) {
+        fill(nxt, k + 1);
+        if (k + 2 < run) issue_loads(k + 2);
       }
-      __syncthreads();  // barrier 2 it + 2: next block visible; output of this block staged
+      __syncthreads();  // second barrier: next block visible; output of this block staged
     }
-    store_out(smem + ((nblk - 1) & 1) * WS_SET, blk0 + (nblk - 1) * step);
+    store_out(smem + ((run - 1) & 1) * WS_SET, first_blk + (run - 1) * step);
     return;
   }
 
@@ -974,7 +1006,9 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
               *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * F) * sizeof(float)));
       }
   };
-  if (SRC == SRC_SCANNED) {
+  if (SRC == SRC_WALK) {
+    if (take_carry) add_state(carry_in + (int64_t)sw.bh * (F * F), 0.f);
+  } else if (SRC == SRC_SCANNED) {
     if (states) {
       // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
       // the segment visited before it (the chunk's incoming state for the first one)
@@ -1020,9 +1054,33 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       }
     }
   }
+  // St <- l^64 St + (scaled Y)^T Z from the feature-major tiles of `set`
+  auto update_state = [&](const char *set, const u32x4 (&zf)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int T = 0; T < 4; ++T)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+    u32x4 yf[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int T = 0; T < 4; ++T) yf[u][T] = lds16(set + WS_YT + tr_off(32 * T + c, 2 * u + hh));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int T = 0; T < 4; ++T) st[T] = E::mfma(yf[u][T], zf[u], st[T]);
+  };
   __syncthreads();  // barrier 0
+  for (int k = 0; k < runup; ++k) {  // walk
+    const char *set = smem + (k & 1) * WS_SET;
+    u32x4 zf[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) zf[u] = lds16(set + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
+    update_state(set, zf);
+    __syncthreads();  // walk barrier k
+  }
   for (int it = 0; it < nblk; ++it) {
-    char *cur = smem + (it & 1) * WS_SET;
+    char *cur = smem + ((runup + it) & 1) * WS_SET;
     // state term, transposed: acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
     floatx16 acc[2];
 #pragma unroll
@@ -1061,11 +1119,6 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       u32x4 zf[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) zf[u] = lds16(cur + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
-      // the state has been consumed by the state term: decay it ahead of the update
-#pragma unroll
-      for (int T = 0; T < 4; ++T)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
       // intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -1075,16 +1128,7 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
           if (needed)
             acc[I] = E::mfma(zf[u], lds16(smem + WS_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2), acc[I]);
         }
-      // state update: St <- l^64 St + (scaled Y)^T Z
-      u32x4 yf[4][4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int T = 0; T < 4; ++T) yf[u][T] = lds16(cur + WS_YT + tr_off(32 * T + c, 2 * u + hh));
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int T = 0; T < 4; ++T) st[T] = E::mfma(yf[u][T], zf[u], st[T]);
+      update_state(cur, zf);
     }
     // stage the output tile (token-major) in the X region of this block
 #pragma unroll
@@ -1099,7 +1143,7 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     __syncthreads();  // barrier 2 it + 2
   }
   // the segment visited last leaves the chunk's outgoing state
-  if (SRC == SRC_COMBINE && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
+  if (SRC != SRC_SCANNED && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
     float *cp = carry_out + (int64_t)sw.bh * (F * F);
 #pragma unroll
     for (int T = 0; T < 4; ++T)
@@ -1117,6 +1161,41 @@ la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, cons
   // SRC_COMBINE: later segments have more states to gather first, so they are started first
   const int item = SRC == SRC_COMBINE ? g.b * g.h * g.n_seg - 1 - (int)blockIdx.x : (int)blockIdx.x;
   ws_body<E, REV, TRANS, SRC>(X, Y, Z, S, states, Out, g, item, smem, carry_in, carry_out);
+}
+
+// A whole short chunk in one launch on the wave-specialised sweep (placement as la_fused_fwd / la_fused_bwd)
+template <class E>
+__global__ void __launch_bounds__(WS_THREADS, 1)
+la_fused_fwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+                const float *__restrict__ S, const float *__restrict__ kv_in, float *__restrict__ kv_out,
+                elem16_t *__restrict__ O, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int bh = (slot / g.n_seg) * 8 + xcd;
+  if (bh >= g.b * g.h) return;
+  const int item = bh * g.n_seg + (g.n_seg - 1 - slot % g.n_seg);
+  ws_body<E, false, false, SRC_WALK>(Q, K, V, S, nullptr, O, g, item, smem, kv_in, kv_out);
+}
+
+template <class E>
+__global__ void __launch_bounds__(WS_THREADS, 1)
+la_fused_bwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+                const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_in,
+                const float *__restrict__ dkv_in, float *__restrict__ dkv_out, elem16_t *__restrict__ DQ,
+                elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
+  extern __shared__ __align__(16) char smem[];
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int per_bh = 3 * g.n_seg;
+  const int bh = (slot / per_bh) * 8 + xcd;
+  if (bh >= g.b * g.h) return;
+  const int rem = slot % per_bh;
+  const int role = rem % 3, k = rem / 3;  // k-th longest walk of its role
+  if (role == 0)
+    ws_body<E, false, true, SRC_WALK>(DO, V, K, S, nullptr, DQ, g, bh * g.n_seg + g.n_seg - 1 - k, smem, kv_in);
+  else if (role == 1)
+    ws_body<E, true, false, SRC_WALK>(K, Q, DO, S, nullptr, DV, g, bh * g.n_seg + k, smem, dkv_in, dkv_out);
+  else
+    ws_body<E, true, true, SRC_WALK>(V, DO, Q, S, nullptr, DK, g, bh * g.n_seg + k, smem, dkv_in);
 }
 
 // la_bwd3 on the wave-specialised sweep (same triples, same placement)
@@ -1384,6 +1463,48 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
   return launch_state_skipping<E, REV, MODE>(y, z, s, states, g, carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1), st);
 }
 
+template <class E>
+int launch_fused_fwd_ws(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_fused_fwd_ws<E>>(WS_LDS);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * g.n_seg);  // whole groups of 8 (b, h)
+  ProfScope prof(KC_FUSED, st);
+  la_fused_fwd_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, a.s, a.kv_in, a.kv_out,
+                                                         (elem16_t *)a.o, g);
+  return (int)hipGetLastError();
+}
+
+// The backward's three workgroups per segment should fit the chip in one round (one workgroup per CU), and
+// nothing ties its segments to the forward's: no states are handed over on this path.
+Geom fused_bwd_geom(const Geom &g) {
+  Geom gb = g;
+  const int64_t bh = (int64_t)g.b * g.h;
+  int64_t fit = 256 / (3 * bh);  // segments per (b, h) in one round
+  if (fit < 1) fit = 1;
+  if (fit < g.n_seg) {
+    int64_t len = (g.n + fit - 1) / fit;
+    len = ((len + BLK - 1) / BLK) * BLK;
+    gb.seg_len = (int)len;
+    gb.n_seg = (int)((g.n + len - 1) / len);
+  }
+  return gb;
+}
+
+template <class E>
+int launch_fused_bwd_ws(const BwdArgs &a, const Geom &g_fwd, hipStream_t st) {
+  int rc = grant_lds<la_fused_bwd_ws<E>>(WS_LDS);
+  if (rc) return rc;
+  const Geom g = fused_bwd_geom(g_fwd);
+  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * 3 * g.n_seg);
+  ProfScope prof(KC_FUSED, st);
+  la_fused_bwd_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
+                                                         a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
+                                                         (elem16_t *)a.dk, (elem16_t *)a.dv, g);
+  return (int)hipGetLastError();
+}
+
 template <class E, int MODE>
 int launch_fused_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
   int rc = grant_lds<la_fused_fwd<E, MODE>>(APPLY_LDS);
@@ -1420,7 +1541,7 @@ Geom pre_pass_geom(const Geom &g) {
 
 template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return launch_fused_fwd<E, MODE>(a, g, st);
+  if (g.fused) return (MODE == M_ALIGNED && g.ws) ? launch_fused_fwd_ws<E>(a, g, st) : launch_fused_fwd<E, MODE>(a, g, st);
   int rc;
   if constexpr (MODE != M_NARROW) if (g.combine) {  // (narrow rows keep the scan: no registers to spare there)
     // few segments: the pre-pass leaves every segment's own state (the last one's is never read), each
@@ -1449,7 +1570,7 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
 
 template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return launch_fused_bwd<E, MODE>(a, g, st);
+  if (g.fused) return (MODE == M_ALIGNED && g.ws) ? launch_fused_bwd_ws<E>(a, g, st) : launch_fused_bwd<E, MODE>(a, g, st);
   int rc;
   if constexpr (MODE != M_NARROW) if (g.combine) {
     const float *kv_states = a.kv_seg_states;

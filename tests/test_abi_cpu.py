@@ -98,12 +98,17 @@ def test_kernel_path_selection(lib):
     assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_MFMA    # rows read zero-extended
     assert _abi.kernel_path(1, 16, 65536, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC  # not a multiple of 8
     # short 16-bit chunks under the default plan: one launch per direction, no workspace
-    # (few segments: the longest walk over preceding blocks stays within 8 blocks)
+    # (few segments: the longest walk over preceding blocks stays within 8 blocks, or within 16 for the
+    # wave-specialised kernels that full-width heads on whole blocks get)
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED    # 2 x 256 tokens
     assert _abi.kernel_path(2, 12, 512, 128, 64, torch.float16) == _abi.PATH_MFMA_FUSED
     assert _abi.kernel_path(1, 3, 768, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED     # 3 x 256 tokens
-    assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 2 x 1024 tokens
-    assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 8 x 256 tokens
+    assert _abi.kernel_path(2, 12, 1024, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 6 x 192 tokens: walks of 15 blocks
+    assert _abi.kernel_path(2, 12, 1024, 128, 64, torch.bfloat16) == _abi.PATH_MFMA          # narrow rows: 8 blocks at most
+    assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 2 x 1024 tokens: 16 blocks
+    assert _abi.kernel_path(4, 32, 2048 + 8, 128, 128, torch.bfloat16) == _abi.PATH_MFMA     # ragged: 8 blocks at most
+    assert _abi.kernel_path(2, 12, 1536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 6 x 256 tokens: 20 blocks
+    assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 7 x 320 tokens
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.float32) == _abi.PATH_MFMA
     # a state is stored zero-extended to 128 x 128 on the MFMA path, d x e on the generic one
     assert _abi.plan(1, 2, 256, 64, 128, torch.bfloat16, 256)[2] == 2 * 128 * 128 * 4

@@ -35,16 +35,17 @@ def run_abi(inp, s, dev, seg_len=0, cache=False, exact=False):
 
 def mfma_path(b, h, n, dtype, d=128, e=128):
     """The path id of an MFMA-eligible shape under the default plan.  Short 16-bit chunks whose segments
-    are few (longest walk over preceding blocks within 8 blocks) run
-    as one launch per direction; an explicit seg_len, as most tests below pass, always selects the
-    pre-pass / scan / sweep kernels."""
+    are few (longest walk over preceding blocks within 8 blocks; within 16 for full-width heads on whole
+    blocks, which get the wave-specialised kernels) run as one launch per direction; an explicit seg_len,
+    as most tests below pass, always selects the pre-pass / scan / sweep kernels."""
     from lasp_amd import _abi
 
     if dtype == torch.float32 or n > 2048:
         return _abi.PATH_MFMA
     seg_len, n_seg, _ = _abi.plan(b, h, n, d, e, dtype)
     per_seg = seg_len // 64
-    return _abi.PATH_MFMA_FUSED if (n_seg - 1) * per_seg <= 8 else _abi.PATH_MFMA
+    limit = 16 if (d == 128 and e == 128 and n % 64 == 0) else 8
+    return _abi.PATH_MFMA_FUSED if (n_seg - 1) * per_seg <= limit else _abi.PATH_MFMA
 
 
 def test_library_loaded_and_path_selection(gpu_device):
@@ -58,7 +59,8 @@ def test_library_loaded_and_path_selection(gpu_device):
     assert _abi.kernel_path(2, 12, 2047, 128, 128, torch.bfloat16) == _abi.PATH_MFMA       # 8 segments: too long a walk
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 segments
     assert _abi.kernel_path(1, 3, 768, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 3 segments, 8-block walk
-    assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA       # 2 segments of 1024
+    assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 segments of 1024: a 16-block walk
+    assert _abi.kernel_path(4, 32, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA        # narrow rows: 8 blocks at most
     assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC
 
@@ -340,6 +342,8 @@ def test_seeded_random_shapes(gpu_device):
     (2, 4, 640, 128, 128),     # three segments, the last one short
     (1, 3, 768, 128, 128),     # three segments
     (1, 2, 64, 128, 128), (1, 1, 192, 128, 128),
+    (2, 12, 1024, 128, 128),   # wave-specialised form: six segments of 192 tokens, walks of up to 15 blocks
+    (4, 32, 2048, 128, 128),   # two segments of 1024 tokens, a walk of 16 blocks; 3 * 128 * 2 workgroups backwards
     (2, 3, 700, 128, 128), (1, 4, 513, 128, 128), (1, 2, 333, 128, 128), (1, 2, 1, 128, 128),   # ragged lengths
     (2, 12, 512, 128, 64), (1, 3, 700, 64, 96), (2, 2, 321, 48, 16),                              # narrow rows
 ])
