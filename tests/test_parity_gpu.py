@@ -334,6 +334,30 @@ def test_seeded_random_shapes(gpu_device):
         check(got, oracle(inp, s), 1e-4 if dtype == torch.float32 else 2e-2, what=what)
 
 
+def test_seeded_random_shapes_on_the_wave_specialised_kernels(gpu_device):
+    """40 shapes drawn from a fixed seed among those the wave-specialised sweeps serve (16-bit, d = e = 128,
+    whole blocks): 1 to 80 blocks, planned and forced segment lengths from one block upwards -- single-launch,
+    scan-less (up to 4 segments) and scan paths, sweep segments longer than the pre-pass's 2048-token pieces,
+    one-block segments, a short last segment -- with and without incoming states, states kept or recomputed."""
+    import random
+
+    rng = random.Random(20260925)
+    for case in range(40):
+        b, h = rng.choice([1, 2]), rng.randint(1, 6)
+        n = 64 * rng.choice([rng.randint(1, 8), rng.randint(9, 40), rng.randint(41, 80)])
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+        seg = rng.choice([0, 0, 0, 64, 128, 192, 320, 512, 1024, 2048, 4096])
+        state = rng.random() < 0.6
+        s = rng.choice([O.slopes_baseline(h), O.slopes_alibi(h), torch.zeros(h, 1, 1), torch.full((h, 1, 1), 0.02),
+                        torch.full((h, 1, 1), 5.0)])
+        inp = make_inputs(b, h, n, 128, 128, dtype, seed=3000 + case, scale=0.3, state=state, state_std=0.5)
+        what = f"case {case}: b={b} h={h} n={n} {dtype} seg={seg} state={state} slopes={s.flatten().tolist()[:3]}"
+        print(what, flush=True)
+        got = run_abi(inp, s, gpu_device, seg_len=seg, cache=bool(case & 1))
+        assert all(torch.isfinite(v_.float()).all() for v_ in got.values() if v_ is not None)
+        check(got, oracle(inp, s), 2e-2, what=what)
+
+
 # ---------------------------------------------------------------- single-launch path for short chunks
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("state", [False, True])
