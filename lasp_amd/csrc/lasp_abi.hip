@@ -149,9 +149,11 @@ constexpr int kFusedMaxWalkWs = 16;
 // costs what the scan launch saves (b*h = 24, n = 2048: 67 against 69 us per chunk in kernels, 691 against 677 us
 // for the 8-chunk chain replayed from a graph), so the limit stays.
 constexpr int64_t kCombineMaxSeg = 4;
-// Full-width 16-bit heads on a chunk of whole blocks: the shapes the wave-specialised sweeps take.
+// The shapes the wave-specialised sweeps take: every 16-bit shape of the MFMA kernels (a ragged last block and
+// rows narrower than 128 features are instantiations of their own).
 bool ws_shape(int64_t n, int d, int e, int dtype) {
-  return mfma_eligible(d, e, dtype) && d == kMaxFeature && e == kMaxFeature && n % kSegQuantum == 0;
+  (void)n;
+  return mfma_eligible(d, e, dtype);
 }
 bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg_len, int64_t n_seg) {
   if (seg_len_arg != 0 || !mfma_eligible(d, e, dtype) || n > kFusedMaxTokens) return false;
@@ -197,7 +199,7 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
                 n_seg_final <= kCombineMaxSeg) ? 1 : 0;
   // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
   g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg_final >= 2) ? 1 : 0;
-  // full-width 16-bit heads on a chunk of whole blocks take the wave-specialised sweeps
+  // the 16-bit MFMA shapes take the wave-specialised sweeps
   g->ws = ws_shape(n, d, e, dtype) ? 1 : 0;
   // The pre-pass walks a segment serially, and its slow-decay heads walk all of it: beyond 2048 tokens that
   // walk outlasts everything else in the launch (b*h = 16, n = 65536: 71 us at 4096 tokens against 51 at

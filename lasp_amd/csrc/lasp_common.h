@@ -63,7 +63,7 @@ struct Geom {
   int pre_len;  // tokens per segment of the pre-pass and the scan: seg_len, or seg_len / 2^k where long sweep
                 // segments are cut finer for the pre-pass (wave-specialised scan path only)
   int pre_n;    // ceil(n / pre_len): states per (b, h) in the workspace
-  int ws;       // d = e = 128, 16-bit, n a multiple of 64: the sweeps run wave-specialised (ws_body)
+  int ws;       // 16-bit MFMA shapes: the sweeps run wave-specialised (ws_body)
 };
 
 // Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels.  A state is an fp32 sum

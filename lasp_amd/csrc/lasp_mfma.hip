@@ -817,11 +817,16 @@ constexpr int WS_SET = WS_ZT + F * LDT;        // one block's tiles
 constexpr int WS_SC = 2 * WS_SET;              // the score tile
 constexpr int WS_LDS = WS_SC + BLK * LDSC;     // 144 384 B: one workgroup per CU
 
-template <class E, bool REV, bool TRANS, int SRC>
+template <class E, bool REV, bool TRANS, int SRC, int MODE>
 __device__ __forceinline__ void
 ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out, const Geom &g,
-        int item, char *smem, const float *__restrict__ carry_in, float *__restrict__ carry_out = nullptr) {
+        int fa, int fb, int item, char *smem, const float *__restrict__ carry_in,
+        float *__restrict__ carry_out = nullptr) {
+  // M_RAGGED / M_NARROW as in apply_body: one partial last block in the chunk; X and Y rows of fa features, Z and
+  // Out rows of fb (read zero-extended to 128, written back at their own width)
+  constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
+  constexpr bool LEAVES_STATE = SRC != SRC_SCANNED;  // the sweep's final state is the chunk's outgoing one
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -841,11 +846,17 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
   // walk gets to the chunk's end, else from zero.  Blocks are numbered relative to the segment; walk and sweep
   // form one run of runup + nblk blocks, first_blk, first_blk + step, ..., of which the first `runup` only
   // update the state (one barrier each, both groups).
+  const int total_blk = (int)((g.n + BLK - 1) / BLK);  // blocks in the chunk
+  const int seg_blk0 = (int)(sw.tok0 / BLK);           // the segment's first block
+  const int chunk_tail = (int)(g.n - (int64_t)(total_blk - 1) * BLK);
+  // tokens in a block (numbered relative to the segment): a partial block is the chunk's last one
+  auto len_of = [&](int blk) __attribute__((always_inline)) {
+    if (!RAGGED) return BLK;
+    return seg_blk0 + blk == total_blk - 1 ? chunk_tail : BLK;
+  };
   int runup = 0;
   bool take_carry = false;
   if (SRC == SRC_WALK) {
-    const int total_blk = (int)(g.n / BLK);
-    const int seg_blk0 = (int)(sw.tok0 / BLK);
     const int avail = REV ? total_blk - (seg_blk0 + nblk) : seg_blk0;
     int reach = avail;
     if (sl > 0.f) {
@@ -863,11 +874,13 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     const int ftid = tid;  // 0..255
     const LoaderRole xr = x_role(ftid), yr = yz_role(ftid);
     const int chunk = ftid & 15, rowq = ftid >> 4;
-    const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + row0 * F);
-    const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * F);
-    const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * F);
-    u32x4 *Og = reinterpret_cast<u32x4 *>(Out + row0 * F);
-    constexpr int U = F / 4;  // 8-byte units per row
+    const int xw = NARROW ? fa : F, zw = NARROW ? fb : F;  // row widths in elements
+    const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + row0 * xw);
+    const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * xw);
+    const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * zw);
+    u32x4 *Og = reinterpret_cast<u32x4 *>(Out + row0 * zw);
+    const int xu = xw / 4, zu = zw / 4;  // 8-byte units per row
+    const int ou = zw / 8;               // 16-byte units per output row
     float kdec[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -876,25 +889,31 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     }
     const int qI = w >> 1, qJ = w & 1;
     const bool q_active = REV ? !(qI == 1 && qJ == 0) : !(qI == 0 && qJ == 1);
-    const uint32_t x_off = lane_offset(xr, xr.rowq, U), y_off = lane_offset(yr, 4 * yr.rowq, U);
+    const uint32_t x_off = lane_offset(xr, xr.rowq, xu), y_off = lane_offset(yr, 4 * yr.rowq, xu),
+                   z_off = lane_offset(yr, 4 * yr.rowq, zu);
     const PieceMask all = {true, true};
+    const PieceMask x_ok = piece_mask(xr, xu), y_ok = piece_mask(yr, xu), z_ok = piece_mask(yr, zu);
 
     // the block in flight, two 8-byte pieces per row (see LoaderRole)
     u32x4 nx[4], ny[4], nz[4];
     // k: position in the run; walk blocks (k < runup) need no X tile
     auto issue_loads = [&](int k) __attribute__((always_inline)) {
       const int blk = first_blk + k * step;
-      const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * U * 8);
-      const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * U * 8);
-      const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * U * 8);
+      const int len = len_of(blk);  // rows past a partial block's end and pieces past a narrow row's width read as zeros
+      const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * xu * 8);
+      const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * xu * 8);
+      const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * zu * 8);
       if (SRC != SRC_WALK || k >= runup) {
 #pragma unroll
-        for (int it = 0; it < 4; ++it) nx[it] = load_row_pieces(xblk, 16 * it * U * 8, x_off, all, true);
+        for (int it = 0; it < 4; ++it)
+          nx[it] = load_row_pieces(xblk, 16 * it * xu * 8, x_off, NARROW ? x_ok : all,
+                                   !RAGGED || xr.rowq + 16 * it < len);
       }
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        ny[r] = load_row_pieces(yblk, r * U * 8, y_off, all, true);
-        nz[r] = load_row_pieces(zblk, r * U * 8, y_off, all, true);
+        const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
+        ny[r] = load_row_pieces(yblk, r * xu * 8, y_off, NARROW ? y_ok : all, row_ok);
+        nz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
       }
     };
     // writes the block held in nx / ny / nz into a tile set: token-major X and Y, feature-major Y (scaled by the
@@ -908,17 +927,29 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
         for (int r = 0; r < 4; ++r)
           *reinterpret_cast<u32x4 *>(set + WS_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
       }
-      store_transposed<E, true>(set + WS_YT, ny, yr, kdec);
+      const int len = len_of(first_blk + k * step);
+      if (LEAVES_STATE && RAGGED && !REV && len != BLK) {
+        // the chunk's partial last block, going forwards: its tokens sit `len - b` before the chunk end, which
+        // matters here because the state it leaves is the outgoing one
+        float kd[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
+        store_transposed<E, true>(set + WS_YT, ny, yr, kd);
+      } else {
+        store_transposed<E, true>(set + WS_YT, ny, yr, kdec);
+      }
       store_transposed<E, false>(set + WS_ZT, nz, yr, kdec);
     };
     // the output tile staged in `set`'s X region -> global rows of block `blk`
     auto store_out = [&](const char *set, int blk) __attribute__((always_inline)) {
       const int64_t brow = (int64_t)blk * BLK;
+      const int len = len_of(blk);
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const int row = rowq + 16 * r4;
-        __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(set + WS_XN + row * LDN + chunk * 16),
-                                    &Og[(brow + row) * (F / 8) + chunk]);
+        if (!RAGGED || (row < len && (!NARROW || chunk < ou)))
+          __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(set + WS_XN + row * LDN + chunk * 16),
+                                      &Og[(brow + row) * (NARROW ? ou : F / 8) + chunk]);
       }
     };
     // this wave's quadrant of the transposed score tile: sc[4g+r] = y_b . x_a, b = 32qJ+8g+4hh+r, a = 32qI+c
@@ -988,26 +1019,39 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
   for (int T = 0; T < 4; ++T)
 #pragma unroll
     for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
-  // st <- f * st + M, M being the 128 x 128 fp32 matrix at `src` (read transposed by the transposed roles)
-  auto add_state = [&](const float *src, float f) __attribute__((always_inline)) {
+  // M_NARROW: a wave whose 32 columns all lie past the width of Z has nothing to compute (it still takes part in
+  // every barrier); the upper 64 features are skipped as a whole when the rows are no wider
+  const bool wave_active = !NARROW || 32 * w < fb;
+  const bool upper_half = !NARROW || fa > 64;
+  // st <- f * st + M, M being the 128 x 128 fp32 tile whose element (row, col) is src[row * ld + col], or for a
+  // transposed role src[col * ld + row]; `bounded`: src holds only fa x fb (transposed: fb x fa) elements
+  auto add_state_ld = [&](const float *src, int ld, float f, bool bounded) __attribute__((always_inline)) {
     typedef const __attribute__((address_space(1))) float *gmem_f32;
     const uint32_t lane_off =
-        (uint32_t)(TRANS ? (32 * w + c) * F + 4 * hh : 4 * hh * F + 32 * w + c) * (uint32_t)sizeof(float);
+        (uint32_t)(TRANS ? (32 * w + c) * ld + 4 * hh : 4 * hh * ld + 32 * w + c) * (uint32_t)sizeof(float);
+    const bool col_ok = !bounded || 32 * w + c < fb;
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
         const int band = 32 * T + 8 * gq;
-        const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : band * F)));
+        const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : (int64_t)band * ld)));
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          st[T][4 * gq + r] = fmaf(
-              f, st[T][4 * gq + r],
-              *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * F) * sizeof(float)));
+        for (int r = 0; r < 4; ++r) {
+          const bool ok = col_ok && (!bounded || band + 4 * hh + r < fa);
+          const float own =
+              ok ? *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * ld) * sizeof(float)) : 0.f;
+          st[T][4 * gq + r] = fmaf(f, st[T][4 * gq + r], own);
+        }
       }
   };
+  // a state of the workspace (128 x 128, zero beyond fa x fb) / the chunk's incoming state (fa x fb, unpadded)
+  auto add_state = [&](const float *src, float f) __attribute__((always_inline)) { add_state_ld(src, F, f, false); };
+  auto add_carry = [&]() __attribute__((always_inline)) {
+    add_state_ld(carry_in + (int64_t)sw.bh * fa * fb, NARROW ? (TRANS ? fa : fb) : F, 0.f, NARROW);
+  };
   if (SRC == SRC_WALK) {
-    if (take_carry) add_state(carry_in + (int64_t)sw.bh * (F * F), 0.f);
+    if (take_carry) add_carry();
   } else if (SRC == SRC_SCANNED) {
     if (states) {
       // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
@@ -1018,17 +1062,18 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       const int sub = g.seg_len / g.pre_len;
       const int piece = REV ? min(sw.seg * sub + sub, g.pre_n) - 1 : sw.seg * sub;
       const float *src = states + ((int64_t)sw.bh * g.pre_n + piece) * (F * F);
-      bool have = true;
+      bool from_carry = false;
       if (state_dies_in_segment(S[sw.bh % g.h], g)) {
         const int nb = REV ? piece + 1 : piece - 1;
-        if (nb < 0 || nb >= g.pre_n) {
-          have = carry_in != nullptr;
-          src = carry_in + (int64_t)sw.bh * (F * F);
-        } else {
+        if (nb < 0 || nb >= g.pre_n)
+          from_carry = true;
+        else
           src = states + ((int64_t)sw.bh * g.pre_n + nb) * (F * F);
-        }
       }
-      if (have) add_state(src, 0.f);
+      if (!from_carry)
+        add_state(src, 0.f);
+      else if (carry_in != nullptr)
+        add_carry();
     }
   } else {
     // `states` holds the segments' OWN states.  The scan's recurrence, St <- l^len_j St + own_j over the
@@ -1043,7 +1088,7 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       if (segs < (float)n_before) first = n_before - ((int)segs + 1);
     }
     first = __builtin_amdgcn_readfirstlane(first);
-    if (first == 0 && carry_in) add_state(carry_in + (int64_t)sw.bh * (F * F), 0.f);
+    if (first == 0 && carry_in) add_carry();
     if (states) {
       const float *base = states + (int64_t)sw.bh * g.n_seg * (F * F);
       const float full = decay(sl, (float)g.seg_len);
@@ -1055,32 +1100,49 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     }
   }
   // St <- l^64 St + (scaled Y)^T Z from the feature-major tiles of `set`
-  auto update_state = [&](const char *set, const u32x4 (&zf)[4]) __attribute__((always_inline)) {
+  auto update_state = [&](const char *set, const u32x4 (&zf)[4], float bd) __attribute__((always_inline)) {
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= blockdec;
+      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
     u32x4 yf[4][4];
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int T = 0; T < 4; ++T) yf[u][T] = lds16(set + WS_YT + tr_off(32 * T + c, 2 * u + hh));
+      for (int T = 0; T < 4; ++T)
+        if (T < 2 || upper_half) yf[u][T] = lds16(set + WS_YT + tr_off(32 * T + c, 2 * u + hh));
 #pragma unroll
     for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int T = 0; T < 4; ++T) st[T] = E::mfma(yf[u][T], zf[u], st[T]);
+      for (int T = 0; T < 4; ++T)
+        if (T < 2 || upper_half) st[T] = E::mfma(yf[u][T], zf[u], st[T]);  // state rows past the width of Y stay zero
   };
   __syncthreads();  // barrier 0
   for (int k = 0; k < runup; ++k) {  // walk
     const char *set = smem + (k & 1) * WS_SET;
-    u32x4 zf[4];
+    if (wave_active) {
+      const int len = len_of(first_blk + k * step);
+      u32x4 zf[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) zf[u] = lds16(set + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
-    update_state(set, zf);
+      for (int u = 0; u < 4; ++u) zf[u] = lds16(set + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
+      update_state(set, zf, RAGGED && len != BLK ? decay(sl, (float)len) : blockdec);
+    }
     __syncthreads();  // walk barrier k
   }
   for (int it = 0; it < nblk; ++it) {
     char *cur = smem + ((runup + it) & 1) * WS_SET;
+    // A partial block is the chunk's last one.  Going forwards nothing after it uses the state (but the outgoing
+    // state where the sweep leaves it); going backwards it comes first and the entering state sits `len` (not 64)
+    // tokens ahead.
+    const int len = len_of(blk0 + it * step);
+    float qd[2] = {qdec[0], qdec[1]};
+    float bd = blockdec;
+    if (RAGGED && REV && len != BLK) {
+      qd[0] = decay(sl, (float)max(len - c, 0));
+      qd[1] = decay(sl, (float)max(len - 32 - c, 0));
+      bd = decay(sl, (float)len);
+    }
+    if (LEAVES_STATE && RAGGED && !REV && len != BLK) bd = decay(sl, (float)len);
     // state term, transposed: acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
     floatx16 acc[2];
 #pragma unroll
@@ -1088,18 +1150,20 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
       acc[0][r] = 0.f;
       acc[1][r] = 0.f;
     }
-    {
+    if (wave_active) {
       // all sixteen X fragments are requested before the first product (these waves have the registers for it)
       const char *x0 = cur + WS_XN + c * LDN + hh * 16;
       const char *x1 = x0 + 32 * LDN;
       u32x4 xf[8][2];
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
+        if (ks >= 4 && !upper_half) continue;
         xf[ks][0] = lds16(x0 + ks * 32);
         xf[ks][1] = lds16(x1 + ks * 32);
       }
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
+        if (ks >= 4 && !upper_half) continue;
         const int T = ks >> 1, u = ks & 1;
         u32x4 a;
         a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
@@ -1113,9 +1177,9 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
 #pragma unroll
     for (int I = 0; I < 2; ++I)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[I][r] *= qdec[I];
+      for (int r = 0; r < 16; ++r) acc[I][r] *= qd[I];
     __syncthreads();  // barrier 2 it + 1: score tile complete
-    {
+    if (wave_active) {
       u32x4 zf[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) zf[u] = lds16(cur + WS_ZT + tr_off(32 * w + c, 2 * u + hh));
@@ -1128,9 +1192,10 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
           if (needed)
             acc[I] = E::mfma(zf[u], lds16(smem + WS_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2), acc[I]);
         }
-      update_state(cur, zf);
+      update_state(cur, zf, bd);
     }
     // stage the output tile (token-major) in the X region of this block
+    if (wave_active)
 #pragma unroll
     for (int I = 0; I < 2; ++I)
 #pragma unroll
@@ -1144,15 +1209,19 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
   }
   // the segment visited last leaves the chunk's outgoing state
   if (SRC != SRC_SCANNED && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
-    float *cp = carry_out + (int64_t)sw.bh * (F * F);
+    float *cp = carry_out + (int64_t)sw.bh * fa * fb;
+    const int col = 32 * w + c;
 #pragma unroll
     for (int T = 0; T < 4; ++T)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) cp[(32 * T + 8 * (r >> 2) + 4 * hh + (r & 3)) * F + 32 * w + c] = st[T][r];
+      for (int r = 0; r < 16; ++r) {
+        const int row = 32 * T + 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (!NARROW || (row < fa && col < fb)) cp[row * (NARROW ? fb : F) + col] = st[T][r];
+      }
   }
 }
 
-template <class E, bool REV, bool TRANS, int SRC>
+template <class E, bool REV, bool TRANS, int SRC, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
             const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
@@ -1160,11 +1229,11 @@ la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, cons
   extern __shared__ __align__(16) char smem[];
   // SRC_COMBINE: later segments have more states to gather first, so they are started first
   const int item = SRC == SRC_COMBINE ? g.b * g.h * g.n_seg - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  ws_body<E, REV, TRANS, SRC>(X, Y, Z, S, states, Out, g, item, smem, carry_in, carry_out);
+  ws_body<E, REV, TRANS, SRC, MODE>(X, Y, Z, S, states, Out, g, g.d, g.e, item, smem, carry_in, carry_out);
 }
 
 // A whole short chunk in one launch on the wave-specialised sweep (placement as la_fused_fwd / la_fused_bwd)
-template <class E>
+template <class E, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_fused_fwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
                 const float *__restrict__ S, const float *__restrict__ kv_in, float *__restrict__ kv_out,
@@ -1174,10 +1243,10 @@ la_fused_fwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, 
   const int bh = (slot / g.n_seg) * 8 + xcd;
   if (bh >= g.b * g.h) return;
   const int item = bh * g.n_seg + (g.n_seg - 1 - slot % g.n_seg);
-  ws_body<E, false, false, SRC_WALK>(Q, K, V, S, nullptr, O, g, item, smem, kv_in, kv_out);
+  ws_body<E, false, false, SRC_WALK, MODE>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
 }
 
-template <class E>
+template <class E, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_fused_bwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
                 const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_in,
@@ -1191,15 +1260,17 @@ la_fused_bwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, 
   const int rem = slot % per_bh;
   const int role = rem % 3, k = rem / 3;  // k-th longest walk of its role
   if (role == 0)
-    ws_body<E, false, true, SRC_WALK>(DO, V, K, S, nullptr, DQ, g, bh * g.n_seg + g.n_seg - 1 - k, smem, kv_in);
+    ws_body<E, false, true, SRC_WALK, MODE>(DO, V, K, S, nullptr, DQ, g, g.e, g.d, bh * g.n_seg + g.n_seg - 1 - k, smem,
+                                            kv_in);
   else if (role == 1)
-    ws_body<E, true, false, SRC_WALK>(K, Q, DO, S, nullptr, DV, g, bh * g.n_seg + k, smem, dkv_in, dkv_out);
+    ws_body<E, true, false, SRC_WALK, MODE>(K, Q, DO, S, nullptr, DV, g, g.d, g.e, bh * g.n_seg + k, smem, dkv_in,
+                                            dkv_out);
   else
-    ws_body<E, true, true, SRC_WALK>(V, DO, Q, S, nullptr, DK, g, bh * g.n_seg + k, smem, dkv_in);
+    ws_body<E, true, true, SRC_WALK, MODE>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
 }
 
 // la_bwd3 on the wave-specialised sweep (same triples, same placement)
-template <class E, int SRC>
+template <class E, int SRC, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
 la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
            const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_states,
@@ -1213,11 +1284,11 @@ la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const
   const int item = n_items - 1 - (grp * 8 + (r & 7));
   if (item < 0) return;
   if (role == 0)
-    ws_body<E, false, true, SRC>(DO, V, K, S, kv_states, DQ, g, item, smem, kv_in);
+    ws_body<E, false, true, SRC, MODE>(DO, V, K, S, kv_states, DQ, g, g.e, g.d, item, smem, kv_in);
   else if (role == 1)
-    ws_body<E, true, false, SRC>(K, Q, DO, S, dkv_states, DV, g, item, smem, dkv_in, dkv_out);
+    ws_body<E, true, false, SRC, MODE>(K, Q, DO, S, dkv_states, DV, g, g.d, g.e, item, smem, dkv_in, dkv_out);
   else
-    ws_body<E, true, true, SRC>(V, DO, Q, S, dkv_states, DK, g, item, smem, dkv_in);
+    ws_body<E, true, true, SRC, MODE>(V, DO, Q, S, dkv_states, DK, g, g.e, g.d, item, smem, dkv_in);
 }
 
 // ------------------------------------------------------------------------------
@@ -1416,28 +1487,27 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
-template <class E, bool REV, bool TRANS, int SRC>
+template <class E, bool REV, bool TRANS, int SRC, int MODE>
 int launch_apply_ws(const void *x, const void *y, const void *z, const float *s, const float *states,
                     const float *carry_in, float *carry_out, void *out, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_apply_ws<E, REV, TRANS, SRC>>(WS_LDS);
+  int rc = grant_lds<la_apply_ws<E, REV, TRANS, SRC, MODE>>(WS_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply_ws<E, REV, TRANS, SRC><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
-                                                                      (const elem16_t *)z, s, states, carry_in,
-                                                                      carry_out, (elem16_t *)out, g);
+  la_apply_ws<E, REV, TRANS, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>(
+      (const elem16_t *)x, (const elem16_t *)y, (const elem16_t *)z, s, states, carry_in, carry_out, (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
-template <class E, int SRC>
+template <class E, int SRC, int MODE>
 int launch_bwd3_ws(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                    hipStream_t st) {
-  int rc = grant_lds<la_bwd3_ws<E, SRC>>(WS_LDS);
+  int rc = grant_lds<la_bwd3_ws<E, SRC, MODE>>(WS_LDS);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3_ws<E, SRC><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_bwd3_ws<E, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                          kv_states, dkv_states, a.kv_in, a.dkv_in, a.dkv_out,
                                                          (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
@@ -1463,13 +1533,13 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
   return launch_state_skipping<E, REV, MODE>(y, z, s, states, g, carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1), st);
 }
 
-template <class E>
+template <class E, int MODE>
 int launch_fused_fwd_ws(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_fused_fwd_ws<E>>(WS_LDS);
+  int rc = grant_lds<la_fused_fwd_ws<E, MODE>>(WS_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * g.n_seg);  // whole groups of 8 (b, h)
   ProfScope prof(KC_FUSED, st);
-  la_fused_fwd_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_fused_fwd_ws<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, a.s, a.kv_in, a.kv_out,
                                                          (elem16_t *)a.o, g);
   return (int)hipGetLastError();
@@ -1491,14 +1561,14 @@ Geom fused_bwd_geom(const Geom &g) {
   return gb;
 }
 
-template <class E>
+template <class E, int MODE>
 int launch_fused_bwd_ws(const BwdArgs &a, const Geom &g_fwd, hipStream_t st) {
-  int rc = grant_lds<la_fused_bwd_ws<E>>(WS_LDS);
+  int rc = grant_lds<la_fused_bwd_ws<E, MODE>>(WS_LDS);
   if (rc) return rc;
   const Geom g = fused_bwd_geom(g_fwd);
   const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * 3 * g.n_seg);
   ProfScope prof(KC_FUSED, st);
-  la_fused_bwd_ws<E><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_fused_bwd_ws<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                          a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
                                                          (elem16_t *)a.dk, (elem16_t *)a.dv, g);
@@ -1541,7 +1611,7 @@ Geom pre_pass_geom(const Geom &g) {
 
 template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return (MODE == M_ALIGNED && g.ws) ? launch_fused_fwd_ws<E>(a, g, st) : launch_fused_fwd<E, MODE>(a, g, st);
+  if (g.fused) return g.ws ? launch_fused_fwd_ws<E, MODE>(a, g, st) : launch_fused_fwd<E, MODE>(a, g, st);
   int rc;
   if constexpr (MODE != M_NARROW) if (g.combine) {  // (narrow rows keep the scan: no registers to spare there)
     // few segments: the pre-pass leaves every segment's own state (the last one's is never read), each
@@ -1549,8 +1619,8 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if (g.n_seg > 1 &&
         (rc = launch_state_skipping<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, g.n_seg - 1, st)))
       return rc;
-    if (MODE == M_ALIGNED && g.ws)
-      return launch_apply_ws<E, false, false, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
+    if (g.ws)
+      return launch_apply_ws<E, false, false, SRC_COMBINE, MODE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
                                                            a.kv_in, a.kv_out, a.o, g, st);
     return launch_apply<E, false, false, MODE, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
                                                             a.kv_in, a.kv_out, a.o, g, st);
@@ -1561,8 +1631,8 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, gp, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, gp, 0, st))) return rc;
   }
-  if (MODE == M_ALIGNED && g.ws)
-    return launch_apply_ws<E, false, false, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
+  if (g.ws)
+    return launch_apply_ws<E, false, false, SRC_SCANNED, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
                                                          a.kv_in, nullptr, a.o, g, st);
   return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
                                                           a.kv_in, nullptr, a.o, g, st);
@@ -1570,7 +1640,7 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
 
 template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return (MODE == M_ALIGNED && g.ws) ? launch_fused_bwd_ws<E>(a, g, st) : launch_fused_bwd<E, MODE>(a, g, st);
+  if (g.fused) return g.ws ? launch_fused_bwd_ws<E, MODE>(a, g, st) : launch_fused_bwd<E, MODE>(a, g, st);
   int rc;
   if constexpr (MODE != M_NARROW) if (g.combine) {
     const float *kv_states = a.kv_seg_states;
@@ -1579,8 +1649,8 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
       kv_states = a.ws_kv;
     }
     if (g.n_seg > 1 && (rc = launch_state_skipping<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, 0, st))) return rc;
-    if (MODE == M_ALIGNED && g.ws)
-      return launch_bwd3_ws<E, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
+    if (g.ws)
+      return launch_bwd3_ws<E, SRC_COMBINE, MODE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
     return launch_bwd3<E, MODE, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g,
                                              st);
   }
@@ -1597,7 +1667,7 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, gp, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  if (MODE == M_ALIGNED && g.ws) return launch_bwd3_ws<E, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
+  if (g.ws) return launch_bwd3_ws<E, SRC_SCANNED, MODE>(a, kv_states, dkv_states, g, st);
   return launch_bwd3<E, MODE, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
 }
 

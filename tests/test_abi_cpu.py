@@ -53,9 +53,10 @@ def test_plan_defaults_and_overrides(lib):
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 4096) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 2048) == (2048, 32, 16 * 32 * 128 * 128 * 4)
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 8192) == (8192, 8, 16 * 32 * 128 * 128 * 4)
-    # ragged or narrow rows stay on the two-per-CU kernels and their plan
+    # ragged lengths and narrow rows are planned like the full-width shapes (15 segments of 4608 tokens would
+    # leave CUs idle, so the ragged length keeps 29)
     assert _abi.plan(1, 16, 65536 + 8, 128, 128, torch.bfloat16)[:2] == (2304, 29)
-    assert _abi.plan(1, 16, 65536, 128, 64, torch.bfloat16) == (2048, 32, 16 * 32 * 128 * 128 * 4)
+    assert _abi.plan(1, 16, 65536, 128, 64, torch.bfloat16) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     # short chunk: 256 tokens per segment at least ...
     assert _abi.plan(1, 16, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
     # ... or 192 where even the backward's 3 workgroups per segment leave the chip under-filled
@@ -98,15 +99,14 @@ def test_kernel_path_selection(lib):
     assert _abi.kernel_path(1, 16, 65536, 64, 128, torch.bfloat16) == _abi.PATH_MFMA    # rows read zero-extended
     assert _abi.kernel_path(1, 16, 65536, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC  # not a multiple of 8
     # short 16-bit chunks under the default plan: one launch per direction, no workspace
-    # (few segments: the longest walk over preceding blocks stays within 8 blocks, or within 16 for the
-    # wave-specialised kernels that full-width heads on whole blocks get)
+    # (few segments: the longest walk over preceding blocks stays within 16 blocks)
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED    # 2 x 256 tokens
     assert _abi.kernel_path(2, 12, 512, 128, 64, torch.float16) == _abi.PATH_MFMA_FUSED
     assert _abi.kernel_path(1, 3, 768, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED     # 3 x 256 tokens
     assert _abi.kernel_path(2, 12, 1024, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 6 x 192 tokens: walks of 15 blocks
-    assert _abi.kernel_path(2, 12, 1024, 128, 64, torch.bfloat16) == _abi.PATH_MFMA          # narrow rows: 8 blocks at most
+    assert _abi.kernel_path(2, 12, 1024, 128, 64, torch.bfloat16) == _abi.PATH_MFMA_FUSED    # narrow rows alike
     assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 2 x 1024 tokens: 16 blocks
-    assert _abi.kernel_path(4, 32, 2048 + 8, 128, 128, torch.bfloat16) == _abi.PATH_MFMA     # ragged: 8 blocks at most
+    assert _abi.kernel_path(4, 32, 2048 + 8, 128, 128, torch.bfloat16) == _abi.PATH_MFMA     # ragged: 3 segments, 32 blocks
     assert _abi.kernel_path(2, 12, 1536, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 6 x 256 tokens: 20 blocks
     assert _abi.kernel_path(2, 12, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA         # 7 x 320 tokens
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.float32) == _abi.PATH_MFMA

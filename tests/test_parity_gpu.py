@@ -35,8 +35,7 @@ def run_abi(inp, s, dev, seg_len=0, cache=False, exact=False):
 
 def mfma_path(b, h, n, dtype, d=128, e=128):
     """The path id of an MFMA-eligible shape under the default plan.  Short 16-bit chunks whose segments
-    are few (longest walk over preceding blocks within 8 blocks; within 16 for full-width heads on whole
-    blocks, which get the wave-specialised kernels) run as one launch per direction; an explicit seg_len,
+    are few (longest walk over preceding blocks within 16 blocks) run as one launch per direction; an explicit seg_len,
     as most tests below pass, always selects the pre-pass / scan / sweep kernels."""
     from lasp_amd import _abi
 
@@ -44,8 +43,7 @@ def mfma_path(b, h, n, dtype, d=128, e=128):
         return _abi.PATH_MFMA
     seg_len, n_seg, _ = _abi.plan(b, h, n, d, e, dtype)
     per_seg = seg_len // 64
-    limit = 16 if (d == 128 and e == 128 and n % 64 == 0) else 8
-    return _abi.PATH_MFMA_FUSED if (n_seg - 1) * per_seg <= limit else _abi.PATH_MFMA
+    return _abi.PATH_MFMA_FUSED if (n_seg - 1) * per_seg <= 16 else _abi.PATH_MFMA
 
 
 def test_library_loaded_and_path_selection(gpu_device):
@@ -60,7 +58,7 @@ def test_library_loaded_and_path_selection(gpu_device):
     assert _abi.kernel_path(2, 12, 512, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 segments
     assert _abi.kernel_path(1, 3, 768, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED   # 3 segments, 8-block walk
     assert _abi.kernel_path(4, 32, 2048, 128, 128, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # 2 segments of 1024: a 16-block walk
-    assert _abi.kernel_path(4, 32, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA        # narrow rows: 8 blocks at most
+    assert _abi.kernel_path(4, 32, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA_FUSED  # narrow rows alike
     assert _abi.kernel_path(2, 12, 2048, 128, 64, torch.bfloat16) == _abi.PATH_MFMA
     assert _abi.kernel_path(2, 12, 2048, 128, 60, torch.bfloat16) == _abi.PATH_GENERIC
 
