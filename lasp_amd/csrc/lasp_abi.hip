@@ -128,18 +128,15 @@ bool mfma_f32_eligible(int d, int e, int dtype) {
 
 // Short chunks given to the library with the default plan run as ONE launch per direction: every
 // workgroup rebuilds the state entering its segment by walking the blocks before it, which saves
-// the pre-pass, its launch and the workspace.  The walk is serial work on the critical path (about
-// 1.3 us per 64-token block against 4-5 us for a block of the sweep), so the path is only taken
-// while the longest walk stays within 8 blocks: measured at b*h = 24 it wins up to n = 512 (49
-// against 53 us forward + backward) and loses beyond.  An explicit seg_len always selects the
-// pre-pass / sweep kernels.
+// the pre-pass, its launch and the workspace.  The walk is serial work on the critical path (0.7 us
+// per 64-token block: the math waves multiply a block into the state while the feed waves fetch and
+// transpose the next one), and the single launch wins up to walks of about 16 blocks.  Forward +
+// backward replayed from a graph over rotating inputs, scan path against single launch: b*h = 24:
+// n = 512 44 / 33 us, 768 48 / 40, 1024 59 / 46, 1536 70 / 69, 2048 81 / 87; b*h = 128, n = 1024:
+// 172 / 133; b*h = 16, n = 2048: 66 / 76; b*h = 4, n = 2048: 45 / 70.  An explicit seg_len always
+// selects the pre-pass / sweep kernels.
 constexpr int64_t kFusedMaxTokens = 2048;
-constexpr int kFusedMaxWalk = 8;  // blocks
-// In the wave-specialised form a walk step costs 0.7 us (other waves fetch and transpose the next block meanwhile),
-// and the single launch wins up to walks of about 16 blocks.  Forward + backward replayed from a graph over
-// rotating inputs, scan path against single launch: b*h = 24: n = 512 44 / 33 us, 768 48 / 40, 1024 59 / 46,
-// 1536 70 / 69, 2048 81 / 87; b*h = 128, n = 1024: 172 / 133; b*h = 16, n = 2048: 66 / 76; b*h = 4, n = 2048: 45 / 70.
-constexpr int kFusedMaxWalkWs = 16;
+constexpr int kFusedMaxWalk = 16;  // blocks
 // With few segments the 16-bit sweeps of full-width heads gather the segments' own states themselves
 // (each workgroup re-runs the scan's recurrence over at most kCombineMaxSeg - 1 states of 64 KiB)
 // and the scan launch is dropped; with one segment the pre-pass goes too.  Measured at b*h = 24,
@@ -149,16 +146,10 @@ constexpr int kFusedMaxWalkWs = 16;
 // costs what the scan launch saves (b*h = 24, n = 2048: 67 against 69 us per chunk in kernels, 691 against 677 us
 // for the 8-chunk chain replayed from a graph), so the limit stays.
 constexpr int64_t kCombineMaxSeg = 4;
-// The shapes the wave-specialised sweeps take: every 16-bit shape of the MFMA kernels (a ragged last block and
-// rows narrower than 128 features are instantiations of their own).
-bool ws_shape(int64_t n, int d, int e, int dtype) {
-  (void)n;
-  return mfma_eligible(d, e, dtype);
-}
 bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg_len, int64_t n_seg) {
   if (seg_len_arg != 0 || !mfma_eligible(d, e, dtype) || n > kFusedMaxTokens) return false;
   const int per_seg = seg_len / kSegQuantum;  // blocks in one segment's sweep
-  return (n_seg - 1) * per_seg <= (ws_shape(n, d, e, dtype) ? kFusedMaxWalkWs : kFusedMaxWalk);
+  return (n_seg - 1) * per_seg <= kFusedMaxWalk;
 }
 
 int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
@@ -176,9 +167,9 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     set_error("too many segments (%lld) for seg_len=%d", (long long)n_seg, seg_len);
     return LASP_E_SEGMENT;
   }
-  const bool ws = ws_shape(n, d, e, dtype) && !fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg);
-  if (ws && seg_len_arg == 0 && n_seg > kCombineMaxSeg) {
-    // The wave-specialised sweeps hold a CU each, so the default plan aims at one round of 256 workgroups in the
+  const bool sweeps16 = mfma_eligible(d, e, dtype) && !fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg);
+  if (sweeps16 && seg_len_arg == 0 && n_seg > kCombineMaxSeg) {
+    // The 16-bit sweeps hold a CU each, so the default plan aims at one round of 256 workgroups in the
     // forward sweep rather than two per CU: longer segments mean fewer states to load and carry (b*h = 16,
     // n = 65536: 4096-token segments, sweeps 193 + 496 us against 201 + 513 with 2048; b*h = 32, n = 16384:
     // 2048 against 1024, 97 + 248 against 102 + 256).
@@ -199,15 +190,13 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
                 n_seg_final <= kCombineMaxSeg) ? 1 : 0;
   // heads whose state dies within a segment skip the scan (16-bit MFMA kernels on the pre-pass / scan / sweep path)
   g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg_final >= 2) ? 1 : 0;
-  // the 16-bit MFMA shapes take the wave-specialised sweeps
-  g->ws = ws_shape(n, d, e, dtype) ? 1 : 0;
   // The pre-pass walks a segment serially, and its slow-decay heads walk all of it: beyond 2048 tokens that
   // walk outlasts everything else in the launch (b*h = 16, n = 65536: 71 us at 4096 tokens against 51 at
   // 2048; at 1024 the extra states cost more again, 62 us and a longer scan).  Long sweep segments are therefore cut in halves (quarters, ...) for the pre-pass and the scan, and
   // a sweep takes the state that enters its first piece.  A pure function of the shape and seg_len, so that a
   // backward call given the forward's seg_len finds the states where the forward left them.
   g->pre_len = seg_len;
-  if (g->ws && !g->combine && !g->fused) {
+  if (mfma_eligible(d, e, dtype) && !g->combine && !g->fused) {
     int pre = seg_len;
     while (pre > kPreMaxSeg && pre % (2 * kSegQuantum) == 0) pre /= 2;
     if (pre <= kPreMaxSeg) g->pre_len = pre;

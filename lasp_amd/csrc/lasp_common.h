@@ -61,9 +61,8 @@ struct Geom {
   int combine;  // few segments: no scan launch, the sweep workgroups gather the segments' own states
   int bypass;   // the scan leaves out heads whose state dies within one segment (see state_dies_in_segment)
   int pre_len;  // tokens per segment of the pre-pass and the scan: seg_len, or seg_len / 2^k where long sweep
-                // segments are cut finer for the pre-pass (wave-specialised scan path only)
+                // segments are cut finer for the pre-pass (16-bit scan path only)
   int pre_n;    // ceil(n / pre_len): states per (b, h) in the workspace
-  int ws;       // 16-bit MFMA shapes: the sweeps run wave-specialised (ws_body)
 };
 
 // Decay weights below 2^-kSkipLog2 are treated as zero by the 16-bit MFMA kernels.  A state is an fp32 sum

@@ -3,7 +3,7 @@
 // (one partial last block) and M_NARROW (rows of d, e < 128 features, multiples of 8, read
 // zero-extended to 128 and written back at their own width; any chunk length).
 //
-// One kernel, `la_apply`, evaluates a causal (or anti-causal) decayed linear
+// One device routine, `ws_body`, evaluates a causal (or anti-causal) decayed linear
 // attention over a segment of 64-token blocks given the state entering it:
 //
 //   causal       out_a = sum_{b<=a} l^(a-b) (x_a . y_b) z_b + l^a      x_a St
@@ -20,11 +20,11 @@
 // `la_seg_state` computes a segment's own contribution to St (the pre-pass whose
 // results the decayed scan stitches together).
 //
-// Work split inside a 256-thread workgroup (4 waves): wave w owns columns
-// [32w, 32w+32) of St and of the output, as four 32x32 fp32 MFMA accumulator
-// tiles that never leave registers; the 64x64 score tile is computed once,
-// cooperatively (one 32x32 quadrant per wave), masked, rounded to 16 bits and shared
-// through LDS.  All products are arranged so that an accumulator tile can be fed
+// Work split inside a 512-thread workgroup (8 waves, one workgroup per CU): four "math"
+// waves own the state and the output -- wave w columns [32w, 32w+32), as four 32x32 fp32
+// MFMA accumulator tiles that never leave registers -- and four "feed" waves fetch and
+// transpose the next block, compute the 64x64 score tile (one 32x32 quadrant per wave;
+// masked, rounded to 16 bits and shared through LDS) and store the outputs.  All products are arranged so that an accumulator tile can be fed
 // back as an MFMA operand without a shuffle: v_mfma_f32_32x32x16_bf16 leaves
 // C[8g+4hh+r][c] in register 4g+r of lane (c, hh) -- four consecutive rows per
 // lane -- and the contraction index of the following product is permuted to
@@ -48,20 +48,13 @@ typedef uint16_t elem16_t;  // raw bits of one bf16 or fp16 element
 
 constexpr int F = 128;      // feature size (d = e)
 constexpr int BLK = 64;     // tokens per block
-constexpr int NTHR = 256;
 constexpr int LDN = 272;    // bytes per row of a token-major tile (256 + 16: rows shift 4 banks)
 constexpr int LDT = 128;    // bytes per row of a feature-major tile (64 tokens), XOR-swizzled
 constexpr int LDSC = 144;   // bytes per row of the score tile (128 + 16)
-constexpr int OFF_XN = 0;
-constexpr int OFF_YN = OFF_XN + BLK * LDN;
-constexpr int OFF_YT = OFF_YN + BLK * LDN;
-constexpr int OFF_ZT = OFF_YT + F * LDT;
-constexpr int OFF_SC = OFF_ZT + F * LDT;
-constexpr int APPLY_LDS = OFF_SC + BLK * LDSC;  // 76800 B: two workgroups per CU
 constexpr float LOG2E = kLog2e;
 constexpr float SKIP_LOG2 = kSkipLog2;  // decay weights below 2^-SKIP_LOG2 are treated as zero (see la_seg_state)
 enum Mode { M_ALIGNED = 0, M_RAGGED = 1, M_NARROW = 2 };
-// where a sweep takes the state entering its segment from (see apply_body)
+// where a sweep takes the state entering its segment from (see ws_body)
 enum Source { SRC_SCANNED = 0, SRC_WALK = 1, SRC_COMBINE = 2 };
 
 // Element policies: the kernels move 16-bit elements as raw bits and only touch their value
@@ -106,12 +99,6 @@ __device__ __forceinline__ gmem_ptr uniform_ptr(const char *p) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
   const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
   return (gmem_ptr)(((uint64_t)hi << 32) | lo);
-}
-
-// The lane's index within its wave, read from the hardware lane counter: two instructions, and no
-// register has to carry it from the top of the kernel to the place that needs it.
-__device__ __forceinline__ int fresh_lane() {
-  return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
 
 __device__ __forceinline__ u32x4 lds16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
@@ -270,11 +257,15 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 }
 
 // ------------------------------------------------------------------------------
-// M_RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
-// partial.  M_NARROW: in addition X and Y rows hold `fa` features, Z and Out rows `fb`
-// (multiples of 8, at most 128); the upper half of the feature steps and state tiles, and waves
-// whose columns lie in the zero extension, are skipped when they would only see zeros.
-// M_ALIGNED carries none of that bookkeeping; fa and fb are read in M_NARROW only.
+// Every sweep kernel below is an instance of ws_body<E, REV, TRANS, SRC, MODE>.
+//
+// MODE.  M_RAGGED: the chunk length is not a multiple of 64, so the last block of the last segment is
+// partial (rows past its end read as zeros, stores are masked, and the decay factors of that one block use
+// its true length).  M_NARROW: in addition X and Y rows hold `fa` features, Z and Out rows `fb`
+// (multiples of 8, at most 128), read zero-extended to 128 and written back at their own width; the upper
+// half of the feature steps and state tiles, and waves whose columns lie in the zero extension, are skipped
+// when they would only see zeros.  M_ALIGNED carries none of that bookkeeping; fa and fb are read in
+// M_NARROW only.
 //
 // SRC says where the state entering the segment comes from.
 // SRC_SCANNED: `states` holds it, left there by the decayed scan over the segments' own states.
@@ -289,515 +280,11 @@ __device__ __forceinline__ SegWork seg_work(const Geom &g, int item) {
 //   repeated walks make it a tool for short chunks.
 // In the last two the workgroup of the segment visited last writes the state it ends with to
 // `carry_out` (non-transposed roles only).
-template <class E, bool REV, bool TRANS, int MODE, int SRC = SRC_SCANNED>
-__device__ __forceinline__ void
-apply_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
-           const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out,
-           const Geom &g, int fa, int fb, int item, char *smem, const float *__restrict__ carry_in = nullptr,
-           float *__restrict__ carry_out = nullptr) {
-  constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
-  constexpr bool FUSED = SRC == SRC_WALK;          // the state walk and its block numbering
-  constexpr bool LEAVES_STATE = SRC != SRC_SCANNED;  // the sweep's final state is the chunk's outgoing one
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
-  const int c = lane & 31, hh = lane >> 5;
-  const LoaderRole xr = x_role(tid), yr = yz_role(tid);
-  const int chunk = tid & 15, rowq = tid >> 4;  // output copy role: 16-byte column, row
-
-  const SegWork sw = seg_work(g, item);
-  const float sl = S[sw.bh % g.h] * LOG2E;
-  const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;  // first row of the segment
-  const int xw = NARROW ? fa : F, zw = NARROW ? fb : F;  // row widths in elements
-  const u32x2 *Xg = reinterpret_cast<const u32x2 *>(X + row0 * xw);
-  const u32x2 *Yg = reinterpret_cast<const u32x2 *>(Y + row0 * xw);
-  const u32x2 *Zg = reinterpret_cast<const u32x2 *>(Z + row0 * zw);
-  u32x4 *Og = reinterpret_cast<u32x4 *>(Out + row0 * zw);
-  const int xu = xw / 4, zu = zw / 4;  // 8-byte units per row
-  const int ou = zw / 8;               // 16-byte units per output row
-
-  // ---- constants (all exponents <= 0)
-  const float blockdec = decay(sl, (float)BLK);
-  float qdec[2];
-#pragma unroll
-  for (int I = 0; I < 2; ++I) {
-    const int a = 32 * I + c;
-    qdec[I] = decay(sl, REV ? (float)(BLK - a) : (float)a);
-  }
-  float kdec[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int b = 4 * yr.rowq + r;
-    kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
-  }
-  // M_NARROW: a wave whose 32 output columns all lie past the width of Z has only its share of
-  // the score tile to compute
-  const bool wave_active = !NARROW || 32 * w < fb;
-  const int qI = w >> 1, qJ = w & 1;  // score quadrant of this wave: queries 32*qI.., keys 32*qJ..
-  const bool q_active = REV ? !(qI == 1 && qJ == 0) : !(qI == 0 && qJ == 1);
-
-  // ---- FUSED: how many blocks outside the segment the state is walked over first
-  const int total_blk = (int)((g.n + BLK - 1) / BLK);          // blocks in the chunk
-  const int seg_blk0 = (int)(sw.tok0 / BLK);                    // the segment's first block
-  const int chunk_tail = (int)(g.n - (int64_t)(total_blk - 1) * BLK);
-  int runup = 0;
-  bool take_carry = false;
-  if (FUSED) {
-    const int avail = REV ? total_blk - (seg_blk0 + sw.nblk) : seg_blk0;
-    int reach = avail;
-    if (sl > 0.f) {
-      const float x = SKIP_LOG2 / (sl * (float)BLK);  // blocks over which a weight falls to 2^-SKIP_LOG2
-      if (x < (float)avail) reach = (int)x + 1;
-    }
-    runup = __builtin_amdgcn_readfirstlane(min(reach, avail));
-    take_carry = carry_in != nullptr && runup == avail;
-  }
-
-  // ---- state entering the segment, as accumulator tiles: st[T][4g+r] = St[32T+8g+4hh+r][32w+c]
-  floatx16 st[4];
-#pragma unroll
-  for (int T = 0; T < 4; ++T)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) st[T][r] = 0.f;
-
-  // st <- f * st + M, M being the 128 x 128 tile whose element (row, col) is src[row * ld + col], or for a
-  // transposed role src[col * ld + row]; `bounded`: src holds only fa x fb (transposed: fb x fa) elements,
-  // the rest of the tile is zero.  Addresses: a scalar pointer per 8-row band (SALU arithmetic) + one
-  // per-lane offset + an immediate.  (The transposed role's loads are scattered, one 128-byte line per lane;
-  // fetching the matrix coalesced into LDS and reading it back transposed was measured and is no faster:
-  // the loads happen once per workgroup and hide behind the other workgroups' streaming.)
-  auto add_state = [&](const float *src, int ld, float f, bool bounded) __attribute__((always_inline)) {
-    typedef const __attribute__((address_space(1))) float *gmem_f32;
-    const uint32_t lane_off =
-        (uint32_t)(TRANS ? (32 * w + c) * ld + 4 * hh : 4 * hh * ld + 32 * w + c) * (uint32_t)sizeof(float);
-    const bool col_ok = !bounded || 32 * w + c < fb;
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
-        const int band = 32 * T + 8 * gq;  // rows band .. band + 7 of the state (this lane: + 4 hh + r)
-        const gmem_ptr bp = uniform_ptr(reinterpret_cast<const char *>(src + (TRANS ? band : (int64_t)band * ld)));
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const bool ok = col_ok && (!bounded || band + 4 * hh + r < fa);
-          const float own =
-              ok ? *reinterpret_cast<gmem_f32>(bp + lane_off + (uint32_t)(TRANS ? r : r * ld) * sizeof(float)) : 0.f;
-          st[T][4 * gq + r] = fmaf(f, st[T][4 * gq + r], own);
-        }
-      }
-  };
-
-  if (SRC == SRC_COMBINE) take_carry = carry_in != nullptr;
-  if (SRC != SRC_SCANNED && take_carry)
-    add_state(carry_in + (int64_t)sw.bh * fa * fb, TRANS ? fa : fb, 0.f, NARROW);  // fa x fb floats, unpadded
-  if (SRC == SRC_COMBINE) {
-    // the scan's recurrence over the segments before (after) this one, in sweep order; a segment's
-    // own state is weighted relative to that segment's far end, so the running state is first
-    // carried across the segment's length (only the chunk's last segment can be shorter)
-    if (states != nullptr) {
-      const float *base = states + (int64_t)sw.bh * g.n_seg * (F * F);
-      const float full = decay(sl, (float)g.seg_len);
-      const float last = decay(sl, (float)(g.n - (int64_t)(g.n_seg - 1) * g.seg_len));
-      const int n_before = REV ? g.n_seg - 1 - sw.seg : sw.seg;
-      for (int i = 0; i < n_before; ++i) {
-        const int j = REV ? g.n_seg - 1 - i : i;
-        add_state(base + (int64_t)j * (F * F), F, j == g.n_seg - 1 ? last : full, false);
-      }
-    }
-  } else if (SRC == SRC_SCANNED && states) {
-    // Scanned states sit at the segment's own index.  A head the scan leaves out (state_dies_in_segment)
-    // still has the pre-pass's own states there: the state entering this segment is then the own state
-    // of the segment visited before it, or the chunk's incoming state for the first one.
-    const float *src = states + ((int64_t)sw.bh * g.n_seg + sw.seg) * (F * F);
-    int ld = F;
-    bool bounded = false, have = true;
-    if (state_dies_in_segment(S[sw.bh % g.h], g)) {
-      const int nb = REV ? sw.seg + 1 : sw.seg - 1;
-      if (nb < 0 || nb >= g.n_seg) {
-        have = carry_in != nullptr;
-        src = carry_in + (int64_t)sw.bh * fa * fb;  // fa x fb floats, unpadded
-        ld = NARROW ? (TRANS ? fa : fb) : F;
-        bounded = NARROW;
-      } else {
-        src = states + ((int64_t)sw.bh * g.n_seg + nb) * (F * F);
-      }
-    }
-    if (have) add_state(src, ld, 0.f, bounded);
-  }
-
-  // ---- block loader: registers <- global, LDS <- registers
-  u32x4 nx[4], ny[4], nz[4];
-  // M_NARROW addressing: uniform tile and row offsets plus these per-thread constants
-  const uint32_t x_off = lane_offset(xr, xr.rowq, xu), y_off = lane_offset(yr, 4 * yr.rowq, xu),
-                 z_off = lane_offset(yr, 4 * yr.rowq, zu);
-  const PieceMask x_ok = piece_mask(xr, xu), y_ok = piece_mask(yr, xu), z_ok = piece_mask(yr, zu);
-  // a partial block (the end of a ragged chunk) reads its missing rows as zeros
-  // every address is a workgroup-uniform block pointer (scalar registers) plus a per-thread 32-bit
-  // offset and an immediate; rows past a partial block's end and pieces past a narrow row's width
-  // read as zeros
-  // Blocks are numbered relative to the segment (FUSED: negative before it, nblk and up after it).
-  // A partial block is the chunk's last one.
-  auto len_of = [&](int blk) __attribute__((always_inline)) {
-    if (!RAGGED) return BLK;
-    if (!FUSED) return blk == sw.nblk - 1 ? sw.tail : BLK;
-    return seg_blk0 + blk == total_blk - 1 ? chunk_tail : BLK;
-  };
-  auto issue_loads = [&](int blk) __attribute__((always_inline)) {
-    const int len = len_of(blk);
-    const gmem_ptr xblk = uniform_ptr(reinterpret_cast<const char *>(Xg) + (int64_t)blk * BLK * xu * 8);
-    const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)blk * BLK * xu * 8);
-    const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)blk * BLK * zu * 8);
-    const PieceMask all = {true, true};
-#pragma unroll
-    for (int it = 0; it < 4; ++it)
-      nx[it] = load_row_pieces(xblk, 16 * it * xu * 8, x_off, NARROW ? x_ok : all,
-                               !RAGGED || xr.rowq + 16 * it < len);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
-      ny[r] = load_row_pieces(yblk, r * xu * 8, y_off, NARROW ? y_ok : all, row_ok);
-      nz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
-    }
-  };
-  auto fill_lds = [&](int blk) __attribute__((always_inline)) {
-#pragma unroll
-    for (int it = 0; it < 4; ++it)
-      *reinterpret_cast<u32x4 *>(smem + OFF_XN + (xr.rowq + 16 * it) * LDN + (2 * xr.G + xr.j) * 16) = nx[it];
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      *reinterpret_cast<u32x4 *>(smem + OFF_YN + (4 * yr.rowq + r) * LDN + (2 * yr.G + yr.j) * 16) = ny[r];
-    const int len = len_of(blk);
-    if (LEAVES_STATE && RAGGED && !REV && len != BLK) {
-      // the chunk's partial last block, going forwards: its tokens sit `len - b` before the chunk end,
-      // which matters here because the state it leaves is the outgoing one
-      float kd[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
-      store_transposed<E, true>(smem + OFF_YT, ny, yr, kd);
-    } else {
-      store_transposed<E, true>(smem + OFF_YT, ny, yr, kdec);
-    }
-    store_transposed<E, false>(smem + OFF_ZT, nz, yr, kdec);
-  };
-
-  const int step = REV ? -1 : 1;
-  int blk = REV ? sw.nblk - 1 : 0;  // the segment's first block in sweep order
-  issue_loads(blk);  // FUSED: stays in flight during the walk below
-
-  // ---- FUSED: state walk outside the segment: St <- l^len St + (scaled Y)^T Z, nothing else.
-  // A pipeline of its own, shaped like la_seg_state's: two register sets in flight, two LDS
-  // buffers (the second one in the X / Y token-major region, idle here), one barrier per block;
-  // loads past the walk's end repeat its last block so that every wait is exact.
-  if (FUSED && runup > 0) {
-    char *const buf_y[2] = {smem + OFF_YT, smem + OFF_XN};
-    char *const buf_z[2] = {smem + OFF_ZT, smem + OFF_XN + F * LDT};
-    static_assert(2 * F * LDT <= OFF_YT - OFF_XN, "the second walk buffer has to fit the token-major tiles");
-    const int w_first = REV ? sw.nblk - 1 + runup : -runup;
-    auto walk_blk = [&](int i) __attribute__((always_inline)) { return w_first + min(i, runup - 1) * step; };
-    auto walk_loads = [&](u32x4 (&py)[4], u32x4 (&pz)[4], int wb) __attribute__((always_inline)) {
-      const int len = len_of(wb);
-      const gmem_ptr yblk = uniform_ptr(reinterpret_cast<const char *>(Yg) + (int64_t)wb * BLK * xu * 8);
-      const gmem_ptr zblk = uniform_ptr(reinterpret_cast<const char *>(Zg) + (int64_t)wb * BLK * zu * 8);
-      const PieceMask all = {true, true};
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
-        py[r] = load_row_pieces(yblk, r * xu * 8, y_off, NARROW ? y_ok : all, row_ok);
-        pz[r] = load_row_pieces(zblk, r * zu * 8, z_off, NARROW ? z_ok : all, row_ok);
-      }
-    };
-    auto walk_fill = [&](int b, const u32x4 (&py)[4], const u32x4 (&pz)[4]) __attribute__((always_inline)) {
-      store_transposed<E, true>(buf_y[b], py, yr, kdec);
-      store_transposed<E, false>(buf_z[b], pz, yr, kdec);
-    };
-    auto walk_step = [&](int b, int wb) __attribute__((always_inline)) {
-      const int len = len_of(wb);
-      const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
-#pragma unroll
-      for (int T = 0; T < 4; ++T)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[T][r] *= bd;
-      if (wave_active) {
-        int cc = fresh_lane() & 31;
-        asm volatile("" : "+v"(cc));
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const u32x4 zf = lds16(buf_z[b] + tr_off(32 * w + cc, 2 * u + hh));
-#pragma unroll
-          for (int T = 0; T < 4; ++T)
-            if (!NARROW || T < 2 || fa > 64)
-              st[T] = E::mfma(lds16(buf_y[b] + tr_off(32 * T + cc, 2 * u + hh)), zf, st[T]);
-        }
-      }
-    };
-    u32x4 ya[4], za[4], yb[4], zb[4];
-    walk_loads(ya, za, walk_blk(0));
-    walk_loads(yb, zb, walk_blk(1));
-    walk_fill(0, ya, za);
-    walk_loads(ya, za, walk_blk(2));
-    __syncthreads();
-    for (int i = 0; i < runup; i += 2) {
-      walk_step(0, walk_blk(i));
-      walk_fill(1, yb, zb);
-      walk_loads(yb, zb, walk_blk(i + 3));
-      __syncthreads();
-      if (i + 1 >= runup) break;
-      walk_step(1, walk_blk(i + 1));
-      walk_fill(0, ya, za);
-      walk_loads(ya, za, walk_blk(i + 4));
-      __syncthreads();
-    }
-  }
-  fill_lds(blk);
-  __syncthreads();
-
-  for (int it = 0; it < sw.nblk; ++it, blk += step) {
-    const bool more = it + 1 < sw.nblk;
-    if (more) issue_loads(blk + step);
-    // A partial block is the chunk's last one.  Going forwards nothing after it uses the state
-    // (but the outgoing state of a FUSED launch); going backwards it comes first and the entering
-    // state sits `len` (not 64) tokens ahead.
-    const int len = len_of(blk);
-    float qd[2] = {qdec[0], qdec[1]};
-    float bd = blockdec;
-    if (RAGGED && REV && len != BLK) {
-      qd[0] = decay(sl, (float)max(len - c, 0));
-      qd[1] = decay(sl, (float)max(len - 32 - c, 0));
-      bd = decay(sl, (float)len);
-    }
-    if (LEAVES_STATE && RAGGED && !REV && len != BLK) bd = decay(sl, (float)len);
-
-    // (1) one sweep over the 8 feature steps feeds two products from the same X fragments:
-    //     state term, transposed:  acc[I][4g+r] = sum_f St[f][32w+8g+4hh+r] x_a[f], a = 32I+c
-    //     score quadrant, transposed: sc[4g+r] = y_b . x_a, b = 32qJ+8g+4hh+r, a = 32qI+c
-    floatx16 acc[2], sc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      acc[0][r] = 0.f;
-      acc[1][r] = 0.f;
-      sc[r] = 0.f;
-    }
-    __builtin_amdgcn_s_setprio(1);
-    {
-      const char *x0 = smem + OFF_XN + c * LDN + hh * 16;
-      const char *x1 = x0 + 32 * LDN;
-      const char *ya = smem + OFF_YN + (32 * qJ + c) * LDN + hh * 16;
-      // M_NARROW: the upper 64 features are skipped as a whole when the rows are no wider
-      const bool upper_half = !NARROW || fa > 64;
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        if (ks >= 4 && !upper_half) continue;
-        const int T = ks >> 1, u = ks & 1;
-        const u32x4 xf0 = lds16(x0 + ks * 32);
-        const u32x4 xf1 = lds16(x1 + ks * 32);
-        if (wave_active) {
-          u32x4 a;
-          a.x = E::pack(st[T][8 * u + 0], st[T][8 * u + 1]);
-          a.y = E::pack(st[T][8 * u + 2], st[T][8 * u + 3]);
-          a.z = E::pack(st[T][8 * u + 4], st[T][8 * u + 5]);
-          a.w = E::pack(st[T][8 * u + 6], st[T][8 * u + 7]);
-          acc[0] = E::mfma(a, xf0, acc[0]);
-          acc[1] = E::mfma(a, xf1, acc[1]);
-        }
-        if (q_active) {
-          const u32x4 yf = lds16(ya + ks * 32);
-          sc = E::mfma(yf, qI ? xf1 : xf0, sc);
-        }
-      }
-    }
-    __builtin_amdgcn_s_setprio(0);
-    // (2) mask the quadrant with l^|a-b| (exponents <= 0 only), round it, share it through LDS;
-    //     scale the state term by the query decay
-    if (q_active) {
-      const int a = 32 * qI + c;
-#pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
-        float m[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int b = 32 * qJ + 8 * gq + 4 * hh + r;
-          const int dist = REV ? b - a : a - b;
-          m[r] = dist >= 0 ? sc[4 * gq + r] * decay(sl, (float)dist) : 0.f;
-        }
-        u32x2 o;
-        o.x = E::pack(m[0], m[1]);
-        o.y = E::pack(m[2], m[3]);
-        *reinterpret_cast<u32x2 *>(smem + OFF_SC + a * LDSC + (32 * qJ + 8 * gq + 4 * hh) * 2) = o;
-      }
-    }
-#pragma unroll
-    for (int I = 0; I < 2; ++I)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[I][r] *= qd[I];
-    // the state has been consumed by the sweep: decay it now, ahead of the update in (4)
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) st[T][r] *= bd;
-
-    __syncthreads();  // A: score tile complete; XN / YN no longer read
-
-    // (3) intra-block term: acc[I] += Z^T[32w.., tokens] * score[a][tokens]
-    //     (token step outermost, so that consecutive MFMAs write different accumulators)
-    if (wave_active) {
-      // The swizzled addresses of the feature-major tiles are recomputed for every block (a few
-      // integer operations each) rather than held in some twenty registers for the whole sweep:
-      // the opaque copy of the lane's column keeps the compiler from hoisting them.
-      int cc = fresh_lane() & 31;
-      asm volatile("" : "+v"(cc));
-      u32x4 zf[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) zf[u] = lds16(smem + OFF_ZT + tr_off(32 * w + cc, 2 * u + hh));
-      __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int I = 0; I < 2; ++I) {
-          const bool needed = REV ? (I == 0 || u >= 2) : (I == 1 || u < 2);
-          if (needed) {
-            const u32x4 b = lds16(smem + OFF_SC + (32 * I + c) * LDSC + (16 * u + 8 * hh) * 2);
-            acc[I] = E::mfma(zf[u], b, acc[I]);
-          }
-        }
-
-      // (4) state update: St <- l^64 St + (scaled Y)^T Z   (the decay was applied after the sweep)
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int T = 0; T < 4; ++T)
-          if (!NARROW || T < 2 || fa > 64)  // state rows past the width of Y stay zero
-            st[T] = E::mfma(lds16(smem + OFF_YT + tr_off(32 * T + cc, 2 * u + hh)), zf[u], st[T]);
-
-      __builtin_amdgcn_s_setprio(0);
-    }
-    // (5) stage the output tile (token-major, in the YN region) for coalesced stores
-#pragma unroll
-    for (int I = 0; I < 2; ++I)
-#pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
-        u32x2 o;
-        o.x = E::pack(acc[I][4 * gq + 0], acc[I][4 * gq + 1]);
-        o.y = E::pack(acc[I][4 * gq + 2], acc[I][4 * gq + 3]);
-        *reinterpret_cast<u32x2 *>(smem + OFF_YN + (32 * I + c) * LDN + (32 * w + 8 * gq + 4 * hh) * 2) = o;
-      }
-    __syncthreads();  // B: staged output complete; YT / ZT / score no longer read
-    {
-      const int64_t brow = (int64_t)blk * BLK;
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int row = rowq + 16 * r4;
-        if (!RAGGED || (row < len && (!NARROW || chunk < ou)))
-          __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(smem + OFF_YN + row * LDN + chunk * 16),
-                                      &Og[(brow + row) * (NARROW ? ou : F / 8) + chunk]);
-      }
-    }
-    if (more) {
-      __syncthreads();  // C: staged output consumed
-      fill_lds(blk + step);
-      __syncthreads();  // D: next block visible
-    }
-  }
-
-  // the segment visited last by the chunk's sweep leaves the outgoing state
-  if (LEAVES_STATE && !TRANS && carry_out != nullptr && sw.seg == (REV ? 0 : g.n_seg - 1)) {
-    float *cp = carry_out + (int64_t)sw.bh * fa * fb;
-    // the lane's position is taken afresh from the hardware lane counter, so that nothing but the
-    // state has to stay in registers across the sweep for this epilogue
-    const int ln = fresh_lane();
-    const int col = 32 * w + (ln & 31);
-#pragma unroll
-    for (int T = 0; T < 4; ++T)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = 32 * T + 8 * (r >> 2) + 4 * (ln >> 5) + (r & 3);
-        if (!NARROW || (row < fa && col < fb)) cp[row * fb + col] = st[T][r];
-      }
-  }
-}
-
-template <class E, bool REV, bool TRANS, int MODE, int SRC>
-__global__ void __launch_bounds__(NTHR, 2)
-la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
-         const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
-         float *__restrict__ carry_out, elem16_t *__restrict__ Out, Geom g) {
-  extern __shared__ __align__(16) char smem[];
-  // SRC_COMBINE: later segments have more states to gather first, so they are started first
-  const int item = SRC == SRC_COMBINE ? g.b * g.h * g.n_seg - 1 - (int)blockIdx.x : (int)blockIdx.x;
-  apply_body<E, REV, TRANS, MODE, SRC>(X, Y, Z, S, states, Out, g, g.d, g.e, item, smem, carry_in, carry_out);
-}
-
-// A whole short chunk in one launch: every workgroup rebuilds the state entering its segment
-// (see FUSED above), so there is no pre-pass, no scan and no workspace.
-template <class E, int MODE>
-__global__ void __launch_bounds__(NTHR, 2)
-la_fused_fwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
-             const float *__restrict__ S, const float *__restrict__ kv_in, float *__restrict__ kv_out,
-             elem16_t *__restrict__ O, Geom g) {
-  extern __shared__ __align__(16) char smem[];
-  // Workgroups are dealt to the 8 XCDs round-robin: all segments of one (b, h) go to the same XCD,
-  // whose L2 then serves the repeated walks over that (b, h)'s K and V; later segments, which walk
-  // over more blocks first, are started first.
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int bh = (slot / g.n_seg) * 8 + xcd;
-  if (bh >= g.b * g.h) return;
-  const int item = bh * g.n_seg + (g.n_seg - 1 - slot % g.n_seg);
-  apply_body<E, false, false, MODE, SRC_WALK>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
-}
-
-// roles as in la_bwd3 (the dV role leaves dKV_out); all roles and segments of one (b, h) on one XCD
-template <class E, int MODE>
-__global__ void __launch_bounds__(NTHR, 2)
-la_fused_bwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
-             const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_in,
-             const float *__restrict__ dkv_in, float *__restrict__ dkv_out, elem16_t *__restrict__ DQ,
-             elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
-  extern __shared__ __align__(16) char smem[];
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int per_bh = 3 * g.n_seg;
-  const int bh = (slot / per_bh) * 8 + xcd;
-  if (bh >= g.b * g.h) return;
-  const int rem = slot % per_bh;
-  const int role = rem % 3, k = rem / 3;  // k-th longest walk of its role
-  if (role == 0)  // dQ walks forwards: late segments have the longest walk
-    apply_body<E, false, true, MODE, SRC_WALK>(DO, V, K, S, nullptr, DQ, g, g.e, g.d, bh * g.n_seg + g.n_seg - 1 - k, smem,
-                                           kv_in);
-  else if (role == 1)
-    apply_body<E, true, false, MODE, SRC_WALK>(K, Q, DO, S, nullptr, DV, g, g.d, g.e, bh * g.n_seg + k, smem, dkv_in,
-                                           dkv_out);
-  else
-    apply_body<E, true, true, MODE, SRC_WALK>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
-}
-
-// The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that
-// work on the same (b*h, segment) and therefore read the same Q, K, V, dO blocks;
-// the triple is spread over block indices 8 apart so that all three land on the same
-// XCD (workgroups are dealt to the 8 XCDs round-robin) and share its L2.
-template <class E, int MODE, int SRC>
-__global__ void __launch_bounds__(NTHR, 2)
-la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
-        const elem16_t *__restrict__ DO, const float *__restrict__ S,
-        const float *__restrict__ kv_states, const float *__restrict__ dkv_states,
-        const float *__restrict__ kv_in, const float *__restrict__ dkv_in, float *__restrict__ dkv_out,
-        elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
-  extern __shared__ __align__(16) char smem[];
-  const int n_items = g.b * g.h * g.n_seg;
-  const int grp = blockIdx.x / 24, r = blockIdx.x - grp * 24;
-  const int role = r >> 3;
-  const int item = n_items - 1 - (grp * 8 + (r & 7));
-  if (item < 0) return;
-  if (role == 0)
-    apply_body<E, false, true, MODE, SRC>(DO, V, K, S, kv_states, DQ, g, g.e, g.d, item, smem, kv_in);
-  else if (role == 1)
-    apply_body<E, true, false, MODE, SRC>(K, Q, DO, S, dkv_states, DV, g, g.d, g.e, item, smem, dkv_in, dkv_out);
-  else
-    apply_body<E, true, true, MODE, SRC>(V, DO, Q, S, dkv_states, DK, g, g.e, g.d, item, smem, dkv_in);
-}
-
 // ------------------------------------------------------------------------------
-// The sweep with the work of a block split between two groups of waves (chunk length a multiple of
-// 64, d = e = 128, state taken from the scan).  apply_body runs fill -> products -> store one after the
-// other in every wave, so a workgroup alone on a CU spends most of a block waiting for its own LDS
-// round trips; here 512 threads form one workgroup per CU:
+// The sweep, with the work of a block split between two groups of waves.  A workgroup whose waves all run
+// fill -> products -> store one after the other spends most of a block waiting for its own LDS round trips
+// (measured on such a form of this kernel: 5806 against 3700 clock ticks per block alone on a CU); here 512
+// threads form one workgroup per CU:
 //   waves 0-3 ("feed"): global loads, the LDS tiles of the NEXT block (transposes and decay scaling
 //     included), the masked score tile of the current block, the coalesced output stores;
 //   waves 4-7 ("math"): own the state and the output accumulators (wave 4 + w: columns [32w, 32w + 32)):
@@ -823,8 +310,6 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
         const float *__restrict__ S, const float *__restrict__ states, elem16_t *__restrict__ Out, const Geom &g,
         int fa, int fb, int item, char *smem, const float *__restrict__ carry_in,
         float *__restrict__ carry_out = nullptr) {
-  // M_RAGGED / M_NARROW as in apply_body: one partial last block in the chunk; X and Y rows of fa features, Z and
-  // Out rows of fb (read zero-extended to 128, written back at their own width)
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
   constexpr bool LEAVES_STATE = SRC != SRC_SCANNED;  // the sweep's final state is the chunk's outgoing one
   const int tid = threadIdx.x;
@@ -1054,8 +539,9 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
     if (take_carry) add_carry();
   } else if (SRC == SRC_SCANNED) {
     if (states) {
-      // as in apply_body: the scanned state of this segment, or for a head the scan leaves out the own state of
-      // the segment visited before it (the chunk's incoming state for the first one)
+      // the scanned state of this segment, or for a head the scan leaves out (state_dies_in_segment), whose
+      // own states are still where the pre-pass put them, the own state of the segment visited before it
+      // (the chunk's incoming state for the first one)
       // The workspace holds one state per segment of the pre-pass, of which this sweep segment spans
       // `sub` (a power of two; 1 unless the plan cut long segments finer for the pre-pass): the state that
       // enters it is the one entering its first piece in sweep order.
@@ -1223,7 +709,7 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
 
 template <class E, bool REV, bool TRANS, int SRC, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
-la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
+la_apply(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z,
             const float *__restrict__ S, const float *__restrict__ states, const float *__restrict__ carry_in,
             float *__restrict__ carry_out, elem16_t *__restrict__ Out, Geom g) {
   extern __shared__ __align__(16) char smem[];
@@ -1232,10 +718,13 @@ la_apply_ws(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, cons
   ws_body<E, REV, TRANS, SRC, MODE>(X, Y, Z, S, states, Out, g, g.d, g.e, item, smem, carry_in, carry_out);
 }
 
-// A whole short chunk in one launch on the wave-specialised sweep (placement as la_fused_fwd / la_fused_bwd)
+// A whole short chunk in one launch: every workgroup rebuilds the state entering its segment (SRC_WALK), so
+// there is no pre-pass, no scan and no workspace.  Workgroups are dealt to the 8 XCDs round-robin: all
+// segments of one (b, h) go to the same XCD, whose L2 then serves the repeated walks over that (b, h)'s K
+// and V; later segments, which walk over more blocks first, are started first.
 template <class E, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
-la_fused_fwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+la_fused_fwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
                 const float *__restrict__ S, const float *__restrict__ kv_in, float *__restrict__ kv_out,
                 elem16_t *__restrict__ O, Geom g) {
   extern __shared__ __align__(16) char smem[];
@@ -1246,9 +735,10 @@ la_fused_fwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, 
   ws_body<E, false, false, SRC_WALK, MODE>(Q, K, V, S, nullptr, O, g, g.d, g.e, item, smem, kv_in, kv_out);
 }
 
+// roles as in la_bwd3 (the dV role leaves dKV_out); all roles and segments of one (b, h) on one XCD
 template <class E, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
-la_fused_bwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+la_fused_bwd(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
                 const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_in,
                 const float *__restrict__ dkv_in, float *__restrict__ dkv_out, elem16_t *__restrict__ DQ,
                 elem16_t *__restrict__ DK, elem16_t *__restrict__ DV, Geom g) {
@@ -1269,10 +759,13 @@ la_fused_bwd_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, 
     ws_body<E, true, true, SRC_WALK, MODE>(V, DO, Q, S, nullptr, DK, g, g.e, g.d, bh * g.n_seg + k, smem, dkv_in);
 }
 
-// la_bwd3 on the wave-specialised sweep (same triples, same placement)
+// The three gradients in one launch.  Workgroups come in triples (dQ, dV, dK) that work on the same
+// (b*h, segment) and therefore read the same Q, K, V, dO blocks; the triple is spread over block indices 8
+// apart so that all three land on the same XCD (workgroups are dealt to the 8 XCDs round-robin) and share
+// its L2.
 template <class E, int SRC, int MODE>
 __global__ void __launch_bounds__(WS_THREADS, 1)
-la_bwd3_ws(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
+la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const elem16_t *__restrict__ V,
            const elem16_t *__restrict__ DO, const float *__restrict__ S, const float *__restrict__ kv_states,
            const float *__restrict__ dkv_states, const float *__restrict__ kv_in, const float *__restrict__ dkv_in,
            float *__restrict__ dkv_out, elem16_t *__restrict__ DQ, elem16_t *__restrict__ DK,
@@ -1459,55 +952,27 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   }
 }
 
-template <class E, bool REV, bool TRANS, int MODE, int SRC>
-int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
-                 const float *carry_in, float *carry_out, void *out, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_apply<E, REV, TRANS, MODE, SRC>>(APPLY_LDS);
-  if (rc) return rc;
-  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
-  ProfScope prof(KC_APPLY, st);
-  la_apply<E, REV, TRANS, MODE, SRC><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)x, (const elem16_t *)y,
-                                                                      (const elem16_t *)z, s, states, carry_in,
-                                                                      carry_out, (elem16_t *)out, g);
-  return (int)hipGetLastError();
-}
-
-template <class E, int MODE, int SRC>
-int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
-                hipStream_t st) {
-  int rc = grant_lds<la_bwd3<E, MODE, SRC>>(APPLY_LDS);
-  if (rc) return rc;
-  const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
-  const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
-  ProfScope prof(KC_BWD3, st);
-  la_bwd3<E, MODE, SRC><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
-                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
-                                                         kv_states, dkv_states, a.kv_in, a.dkv_in, a.dkv_out,
-                                                         (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
-  return (int)hipGetLastError();
-}
-
 template <class E, bool REV, bool TRANS, int SRC, int MODE>
-int launch_apply_ws(const void *x, const void *y, const void *z, const float *s, const float *states,
+int launch_apply(const void *x, const void *y, const void *z, const float *s, const float *states,
                     const float *carry_in, float *carry_out, void *out, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_apply_ws<E, REV, TRANS, SRC, MODE>>(WS_LDS);
+  int rc = grant_lds<la_apply<E, REV, TRANS, SRC, MODE>>(WS_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_APPLY, st);
-  la_apply_ws<E, REV, TRANS, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>(
+  la_apply<E, REV, TRANS, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>(
       (const elem16_t *)x, (const elem16_t *)y, (const elem16_t *)z, s, states, carry_in, carry_out, (elem16_t *)out, g);
   return (int)hipGetLastError();
 }
 
 template <class E, int SRC, int MODE>
-int launch_bwd3_ws(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
+int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_states, const Geom &g,
                    hipStream_t st) {
-  int rc = grant_lds<la_bwd3_ws<E, SRC, MODE>>(WS_LDS);
+  int rc = grant_lds<la_bwd3<E, SRC, MODE>>(WS_LDS);
   if (rc) return rc;
   const int64_t n_items = (int64_t)g.b * g.h * g.n_seg;
   const unsigned grid = (unsigned)(((n_items + 7) / 8) * 24);
   ProfScope prof(KC_BWD3, st);
-  la_bwd3_ws<E, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_bwd3<E, SRC, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                          kv_states, dkv_states, a.kv_in, a.dkv_in, a.dkv_out,
                                                          (elem16_t *)a.dq, (elem16_t *)a.dk, (elem16_t *)a.dv, g);
@@ -1534,12 +999,12 @@ int launch_state(const void *y, const void *z, const float *s, float *states, co
 }
 
 template <class E, int MODE>
-int launch_fused_fwd_ws(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_fused_fwd_ws<E, MODE>>(WS_LDS);
+int launch_fused_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
+  int rc = grant_lds<la_fused_fwd<E, MODE>>(WS_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * g.n_seg);  // whole groups of 8 (b, h)
   ProfScope prof(KC_FUSED, st);
-  la_fused_fwd_ws<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_fused_fwd<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, a.s, a.kv_in, a.kv_out,
                                                          (elem16_t *)a.o, g);
   return (int)hipGetLastError();
@@ -1562,38 +1027,13 @@ Geom fused_bwd_geom(const Geom &g) {
 }
 
 template <class E, int MODE>
-int launch_fused_bwd_ws(const BwdArgs &a, const Geom &g_fwd, hipStream_t st) {
-  int rc = grant_lds<la_fused_bwd_ws<E, MODE>>(WS_LDS);
+int launch_fused_bwd(const BwdArgs &a, const Geom &g_fwd, hipStream_t st) {
+  int rc = grant_lds<la_fused_bwd<E, MODE>>(WS_LDS);
   if (rc) return rc;
   const Geom g = fused_bwd_geom(g_fwd);
   const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * 3 * g.n_seg);
   ProfScope prof(KC_FUSED, st);
-  la_fused_bwd_ws<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
-                                                         (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
-                                                         a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
-                                                         (elem16_t *)a.dk, (elem16_t *)a.dv, g);
-  return (int)hipGetLastError();
-}
-
-template <class E, int MODE>
-int launch_fused_fwd(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_fused_fwd<E, MODE>>(APPLY_LDS);
-  if (rc) return rc;
-  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * g.n_seg);  // whole groups of 8 (b, h)
-  ProfScope prof(KC_FUSED, st);
-  la_fused_fwd<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
-                                                         (const elem16_t *)a.v, a.s, a.kv_in, a.kv_out,
-                                                         (elem16_t *)a.o, g);
-  return (int)hipGetLastError();
-}
-
-template <class E, int MODE>
-int launch_fused_bwd(const BwdArgs &a, const Geom &g, hipStream_t st) {
-  int rc = grant_lds<la_fused_bwd<E, MODE>>(APPLY_LDS);
-  if (rc) return rc;
-  const unsigned grid = (unsigned)((((int64_t)g.b * g.h + 7) / 8) * 8 * 3 * g.n_seg);
-  ProfScope prof(KC_FUSED, st);
-  la_fused_bwd<E, MODE><<<grid, NTHR, APPLY_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
+  la_fused_bwd<E, MODE><<<grid, WS_THREADS, WS_LDS, st>>>((const elem16_t *)a.q, (const elem16_t *)a.k,
                                                          (const elem16_t *)a.v, (const elem16_t *)a.d_o, a.s,
                                                          a.kv_in, a.dkv_in, a.dkv_out, (elem16_t *)a.dq,
                                                          (elem16_t *)a.dk, (elem16_t *)a.dv, g);
@@ -1611,19 +1051,16 @@ Geom pre_pass_geom(const Geom &g) {
 
 template <class E, int MODE>
 int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return g.ws ? launch_fused_fwd_ws<E, MODE>(a, g, st) : launch_fused_fwd<E, MODE>(a, g, st);
+  if (g.fused) return launch_fused_fwd<E, MODE>(a, g, st);
   int rc;
-  if constexpr (MODE != M_NARROW) if (g.combine) {  // (narrow rows keep the scan: no registers to spare there)
+  if constexpr (MODE != M_NARROW) if (g.combine) {  // (the plan combines full-width heads only)
     // few segments: the pre-pass leaves every segment's own state (the last one's is never read), each
     // sweep workgroup gathers the ones before it, and the last segment's sweep ends with KV_out
     if (g.n_seg > 1 &&
         (rc = launch_state_skipping<E, false, MODE>(a.k, a.v, a.s, a.seg_states, g, g.n_seg - 1, st)))
       return rc;
-    if (g.ws)
-      return launch_apply_ws<E, false, false, SRC_COMBINE, MODE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
-                                                           a.kv_in, a.kv_out, a.o, g, st);
-    return launch_apply<E, false, false, MODE, SRC_COMBINE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
-                                                            a.kv_in, a.kv_out, a.o, g, st);
+    return launch_apply<E, false, false, SRC_COMBINE, MODE>(a.q, a.k, a.v, a.s, g.n_seg > 1 ? a.seg_states : nullptr,
+                                                               a.kv_in, a.kv_out, a.o, g, st);
   }
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   const Geom gp = pre_pass_geom(g);
@@ -1631,16 +1068,13 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, gp, a.kv_out != nullptr, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, gp, 0, st))) return rc;
   }
-  if (g.ws)
-    return launch_apply_ws<E, false, false, SRC_SCANNED, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
-                                                         a.kv_in, nullptr, a.o, g, st);
-  return launch_apply<E, false, false, MODE, SRC_SCANNED>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
-                                                          a.kv_in, nullptr, a.o, g, st);
+  return launch_apply<E, false, false, SRC_SCANNED, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
+                                                             a.kv_in, nullptr, a.o, g, st);
 }
 
 template <class E, int MODE>
 int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
-  if (g.fused) return g.ws ? launch_fused_bwd_ws<E, MODE>(a, g, st) : launch_fused_bwd<E, MODE>(a, g, st);
+  if (g.fused) return launch_fused_bwd<E, MODE>(a, g, st);
   int rc;
   if constexpr (MODE != M_NARROW) if (g.combine) {
     const float *kv_states = a.kv_seg_states;
@@ -1649,10 +1083,8 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
       kv_states = a.ws_kv;
     }
     if (g.n_seg > 1 && (rc = launch_state_skipping<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, g, 0, st))) return rc;
-    if (g.ws)
-      return launch_bwd3_ws<E, SRC_COMBINE, MODE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
-    return launch_bwd3<E, MODE, SRC_COMBINE>(a, g.n_seg > 1 ? kv_states : nullptr, g.n_seg > 1 ? a.ws_dkv : nullptr, g,
-                                             st);
+    return launch_bwd3<E, SRC_COMBINE, MODE>(a, g.n_seg > 1 ? kv_states : nullptr,
+                                                g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
   }
   const Geom gp = pre_pass_geom(g);
   const float *kv_states = a.kv_seg_states;
@@ -1667,8 +1099,7 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, gp, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
-  if (g.ws) return launch_bwd3_ws<E, SRC_SCANNED, MODE>(a, kv_states, dkv_states, g, st);
-  return launch_bwd3<E, MODE, SRC_SCANNED>(a, kv_states, dkv_states, g, st);
+  return launch_bwd3<E, SRC_SCANNED, MODE>(a, kv_states, dkv_states, g, st);
 }
 
 
