@@ -77,8 +77,8 @@ extern "C" {
                                d = e = 128 */
 #define LASP_PATH_MFMA_FUSED 2 /* short chunks of the 16-bit MFMA shapes called with seg_len = 0 (n <= 2048
                                and few enough segments that rebuilding a segment's incoming state from
-                               the blocks before it -- at most 8 of them, 16 for d = e = 128 and n a
-                               multiple of 64 -- is cheaper than a pre-pass and a scan): one launch
+                               the blocks before it -- at most 16 of them -- is cheaper than a pre-pass
+                               and a scan): one launch
                                per direction; NO workspace is read or written (seg_states,
                                kv_seg_states and workspace may be NULL and are ignored) and the forward
                                leaves no segment states behind.  An explicit seg_len selects
