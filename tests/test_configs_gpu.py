@@ -194,3 +194,42 @@ def _operator_chain(q, k, v, do, s, chunks):
         lasp_amd.destroy_parallel_groups()
     return dict(o=torch.cat([o.detach() for o in outs], 2), dq=torch.cat([l[0].grad for l in leaves], 2),
                 dk=torch.cat([l[1].grad for l in leaves], 2), dv=torch.cat([l[2].grad for l in leaves], 2))
+
+
+def test_headline_shape_ragged_and_narrow_instantiations(gpu_device):
+    """The ragged-length and narrow-row instantiations of the sweeps at the headline size (16 sweep segments of
+    4096 tokens over 2048-token pieces of the pre-pass), every head, against the aligned full-width kernels:
+    * a chunk of n - 8 tokens equals the first n - 8 tokens of the n-token chunk whose last 8 dO rows are zero
+      (O and dQ are causal; with a zero tail in dO nothing flows back from the cut-off tokens into dK and dV);
+    * rows of 64 features equal the full-width kernels on the same rows zero-extended to 128 (zero columns add
+      nothing to any product)."""
+    from lasp_amd import _abi
+
+    dev = gpu_device
+    b, h, n, d = 1, 16, 65536, 128
+    q, k, v, do = [_randn((b, h, n, d), dev, 230 + i, d ** -0.5) for i in range(4)]
+    s = O.slopes_baseline(h).to(dev)
+    kv = torch.randn(b, h, d, d, device=dev, generator=torch.Generator(device=dev).manual_seed(240))
+    do[:, :, n - 8:] = 0
+    full = _fwd_bwd(q, k, v, do, s, kv=kv)
+    cut = n - 8
+    assert _abi.plan(b, h, cut, d, d, torch.bfloat16)[0] == _abi.plan(b, h, n, d, d, torch.bfloat16)[0] == 4096
+    c = lambda t: t[:, :, :cut].contiguous()
+    ragged = _fwd_bwd(c(q), c(k), c(v), c(do), s, kv=kv)
+    torch.cuda.synchronize()
+    for name in ("o", "dq", "dk", "dv"):
+        assert _rel(ragged[name], full[name][:, :, :cut]) <= 1e-3, name
+    del ragged, full
+
+    half = lambda t: t[..., :64].contiguous()
+    pad = lambda t: torch.nn.functional.pad(t, (0, 64))
+    qn, kn, vn, don = half(q), half(k), half(v), half(do)
+    kvn = kv[:, :, :64, :64].contiguous()
+    narrow = _fwd_bwd(qn, kn, vn, don, s, kv=kvn)
+    kvw = torch.zeros_like(kv)
+    kvw[:, :, :64, :64] = kvn
+    wide = _fwd_bwd(pad(qn), pad(kn), pad(vn), pad(don), s, kv=kvw)
+    torch.cuda.synchronize()
+    for name in ("o", "dq", "dk", "dv"):
+        assert _rel(narrow[name], wide[name][..., :64]) <= 1e-3, name
+    assert _rel(narrow["kv_out"], wide["kv_out"][:, :, :64, :64]) <= 1e-3
