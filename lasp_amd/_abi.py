@@ -82,6 +82,11 @@ def _raise(rc: int, what: str):
     raise LaspError(f"{what} failed (code {rc}): {msg}")
 
 
+def _raw_stream(dev) -> int:
+    """hipStream_t of torch's current stream on `dev`, as an integer (no Stream object is built on the way)."""
+    return torch._C._cuda_getCurrentRawStream(dev.index)
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else t.data_ptr()
 
@@ -176,7 +181,7 @@ def stream_probe(reads, writes, grid: int) -> None:
     rd = (_c_void_p * max(len(reads), 1))(*[t.data_ptr() for t in reads])
     wr = (_c_void_p * max(len(writes), 1))(*[t.data_ptr() for t in writes])
     rc = lib.lasp_stream_probe(rd, len(reads), wr, len(writes), sizes.pop(), grid,
-                               torch.cuda.current_stream(dev).cuda_stream)
+                               _raw_stream(dev))
     if rc:
         _raise(rc, "lasp_stream_probe")
 
@@ -245,7 +250,7 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
             states = torch.empty((b, h, n_seg, state_bytes // (4 * b * h * n_seg)), dtype=torch.float32, device=dev)
         rc = lib.lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
                                 o.data_ptr(), _ptr(states), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
-                                torch.cuda.current_stream(dev).cuda_stream)
+                                _raw_stream(dev))
     if rc:
         _raise(rc, "lasp_chunk_fwd")
     return o, states, seg_len
@@ -276,7 +281,7 @@ def chunk_fwd_static(q, k, v, s, o, kv_in=None, kv_out=None, seg_len: int = 0) -
     _check_state("kv_out", kv_out, b, h, d, e)
     rc = lib.lasp_chunk_fwd_static(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
                                    o.data_ptr(), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
-                                   torch.cuda.current_stream(dev).cuda_stream)
+                                   _raw_stream(dev))
     if rc:
         _raise(rc, "lasp_chunk_fwd_static")
 
@@ -317,7 +322,7 @@ def _chunk_bwd_exact(q, k, v, s, do, kv_in=None, dkv_in=None, dkv_out=None, kv_s
         rc = lib.lasp_chunk_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), do.data_ptr(), _ptr(kv_in),
                                 _ptr(dkv_in), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _ptr(dkv_out),
                                 _ptr(kv_seg_states), _ptr(ws), n_arrays * state_bytes, b, h, n, d, e,
-                                DTYPE_CODE[q.dtype], seg_len, torch.cuda.current_stream(dev).cuda_stream)
+                                DTYPE_CODE[q.dtype], seg_len, _raw_stream(dev))
     if rc:
         _raise(rc, "lasp_chunk_bwd")
     return dq, dk, dv
