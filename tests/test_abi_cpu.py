@@ -156,8 +156,8 @@ def test_in_place_state_update_rules(lib):
 
 
 def test_documented_launch_shims_run_as_written(lib, monkeypatch):
-    """The reference-side binding shown in INTEGRATION.md (its python blocks, executed as they stand) must get
-    past the library's argument checks on the reference's own per-rank test shape, n = 512, where the kernels
+    """The reference-side binding that the integration notes at the repository root show (their python blocks,
+    executed as they stand) must get past the library's argument checks on the reference's own per-rank test shape, n = 512, where the kernels
     cannot update a state in place: with host tensors the call that stops it is the device check, not
     LASP_E_ALIAS."""
     import contextlib
