@@ -11,7 +11,8 @@
  *     v, o, do, dv : (b, h, n, e)      element type `dtype`
  *     s            : h floats          per-head decay slope, >= 0
  *     kv_in, kv_out, dkv_in, dkv_out : (b, h, d, e) float, may be NULL
- *     seg states   : (b, h, n_seg, d, e) float workspace (see lasp_plan)
+ *     seg states   : float workspace of lasp_plan's state_bytes (one state per (b, h) and segment, or per
+ *                    piece of a long segment; each d x e, or zero-extended to 128 x 128): opaque to the caller
  *
  * Alignment: q, k, v, o, do, dq, dk, dv start on a 16-byte boundary (the kernels
  * fetch rows with 8-byte loads and store them with 16-byte stores; rows of d or e

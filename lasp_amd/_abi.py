@@ -225,8 +225,8 @@ class _on_device:
 def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
     """Enqueues the forward of one chunk.  Returns (o, seg_states, seg_len).
 
-    seg_states is the (b, h, n_seg, d, e) float32 array of states entering each
-    segment (None when the call needed none); pass it to chunk_bwd to skip the
+    seg_states is the float32 array of states entering each segment, sized by
+    lasp_plan (None when the call needed none); pass it to chunk_bwd to skip the
     recompute.
     """
     lib = load()
@@ -246,8 +246,9 @@ def _chunk_fwd_exact(q, k, v, s, kv_in=None, kv_out=None, seg_len: int = 0):
         o = torch.empty((b, h, n, e), dtype=q.dtype, device=dev)
         states = None
         if not fused and (n_seg > 1 or kv_in is not None or kv_out is not None):
-            # the library decides how a state is stored (d x e, or zero-extended to 128 x 128)
-            states = torch.empty((b, h, n_seg, state_bytes // (4 * b * h * n_seg)), dtype=torch.float32, device=dev)
+            # the library decides how many states it keeps (one per segment, or per piece of a long segment)
+            # and how each is stored (d x e, or zero-extended to 128 x 128): the array is opaque here
+            states = torch.empty((state_bytes // 4,), dtype=torch.float32, device=dev)
         rc = lib.lasp_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), s.data_ptr(), _ptr(kv_in), _ptr(kv_out),
                                 o.data_ptr(), _ptr(states), b, h, n, d, e, DTYPE_CODE[q.dtype], seg_len,
                                 _raw_stream(dev))

@@ -434,3 +434,33 @@ def test_fp16_large_incoming_state_stays_finite(gpu_device):
         got = run_abi(inp, s, gpu_device, seg_len=seg)
         assert all(torch.isfinite(v_.float()).all() for v_ in got.values())
         check(got, oracle(inp, s), 2e-2, what=f"fp16 with kv_in of std 1e3, seg={seg}")
+
+
+def test_odd_number_of_pre_pass_pieces(gpu_device):
+    """A long sweep segment is cut in two for the pre-pass, and a chunk may end within the first half of its last
+    segment: the workspace then holds an odd number of states per (b, h), which is not a multiple of the number
+    of sweep segments (the workspace is sized by lasp_plan's state_bytes alone).  Forward + backward with the
+    forward's states kept, against the oracle and against recomputed states."""
+    from lasp_amd import _abi
+
+    dev = gpu_device
+    b, h, n, d = 1, 4, 4096 * 5 - 2048 - 8, 128
+    seg_len, n_seg, state_bytes = _abi.plan(b, h, n, d, d, torch.bfloat16, 4096)
+    assert (seg_len, n_seg) == (4096, 5) and state_bytes == b * h * 9 * d * d * 4
+    inp = make_inputs(b, h, n, d, d, torch.bfloat16, seed=91, scale=d ** -0.5, state=True, device=dev)
+    s = O.slopes_baseline(16).reshape(-1)[[0, 9, 14, 15]].contiguous().to(dev)
+    kv_out, dkv_out = torch.empty_like(inp["kv"]), torch.empty_like(inp["dkv"])
+    o, states, sl = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=kv_out, seg_len=4096)
+    assert states.numel() * 4 == state_bytes
+    kept = _abi.chunk_bwd(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=inp["dkv"],
+                          dkv_out=dkv_out, kv_seg_states=states, seg_len=sl)
+    redone = _abi.chunk_bwd(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=inp["dkv"],
+                            dkv_out=None, kv_seg_states=None, seg_len=sl)
+    torch.cuda.synchronize()
+    for a, r in zip(kept, redone):
+        assert torch.equal(a, r)
+    cpu = {k_: t.cpu() for k_, t in inp.items()}
+    ref = O.ref_chunked(cpu["q"], cpu["k"], cpu["v"], s.cpu(), cpu["do"], cpu["kv"], cpu["dkv"], dtype=torch.float32)
+    got = dict(o=o, dq=kept[0], dk=kept[1], dv=kept[2], kv_out=kv_out, dkv_out=dkv_out)
+    for name, t in got.items():
+        assert O.rel_err(t.cpu(), ref[name]) <= 2e-2, name
