@@ -61,7 +61,10 @@ constexpr int kMinSeg = 256;
 constexpr int kPreferredSeg = 1024;     // preferred lower bound while kMinGroups workgroups remain
 constexpr int64_t kMinGroups = 256;     // one workgroup per CU
 constexpr int64_t kMaxSeg = 1 << 24;    // offsets inside a segment stay within 32 bits
-constexpr int kPreMaxSeg = 2048;        // longest segment the pre-pass walks in one workgroup (see make_geom)
+constexpr int kLongestPlanned = 4352;   // longest segment the refined default plan picks (4096 tokens and a little more)
+constexpr int kPreMaxSeg = 2304;        // longest segment the pre-pass walks in one workgroup (see make_geom):
+                                        // 2048 tokens and a little more, so that lengths just above 4096, 8192, ...
+                                        // are still cut in 2, 4, ... and not in twice as many pieces
 
 int check_shape(int b, int h, int64_t n, int d, int e, int dtype) {
   if (dtype != LASP_DTYPE_F32 && dtype != LASP_DTYPE_BF16 && dtype != LASP_DTYPE_F16) {
@@ -176,6 +179,48 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     while ((int64_t)b * h * ((n + 2 * seg_len - 1) / (2 * seg_len)) >= kMinGroups &&
            (n + 2 * seg_len - 1) / (2 * seg_len) > kCombineMaxSeg)
       seg_len *= 2;
+    // That leaves between one and two rounds of workgroups, and a round that is only part full costs a whole
+    // round's time.  So the plan is refined: of the segment counts that fill r = 1, 2, ... rounds of the forward
+    // sweep (floor(256 r / (b*h)) segments per (b, h), the segments stretched to cover the chunk) and give
+    // segments of 1024 to about 4096 tokens, the one that keeps the most CUs busy -- fill of the last round,
+    // times the share of a full segment that the chunk's last segment has, times the share of a workgroup's time
+    // that goes into blocks -- is taken, fewer rounds winning ties.  Measured forward + backward, this plan against the power-of-two one: b*h = 24, n = 16384: 10
+    // segments of 1664 tokens, 334 us against 356; b*h = 24, n = 32768: 647 against 742 (11 segments of 3072 =
+    // 264 workgroups); b*h = 28, n = 65536: 18 of 3648, 1417 against 1493; b*h = 48, n = 65536: 16 of 4096, 2407
+    // against 2715; b*h = 100, n = 8192: 5 of 1664, 669 against 733.  In a one-round plan lengths beyond 2048
+    // tokens stay a multiple of 64 * 2^k with seg_len / 2^k <= kPreMaxSeg, so that the pre-pass can work on equal
+    // pieces of that length.
+    const int64_t bh = (int64_t)b * h;
+    double best = 0.0;
+    int best_len = 0;
+    for (int r = 1; r <= 16; ++r) {
+      const int64_t fit = kMinGroups * r / bh;  // segments per (b, h) in r rounds
+      if (fit <= kCombineMaxSeg) continue;
+      const int64_t len = (n + fit - 1) / fit;
+      int64_t stretched = 0;
+      if (r > 1) {  // (more than one round: the pre-pass takes whole segments, see pre_len below)
+        stretched = ((len + kSegQuantum - 1) / kSegQuantum) * kSegQuantum;
+      } else {
+        for (int k = 0; k < 16 && !stretched; ++k) {
+          const int64_t gran = (int64_t)kSegQuantum << k;
+          const int64_t cand = ((len + gran - 1) / gran) * gran;
+          if ((cand >> k) <= kPreMaxSeg) stretched = cand;
+        }
+      }
+      if (stretched < kPreferredSeg) break;  // more rounds only make the segments shorter
+      if (stretched > kLongestPlanned) continue;
+      const int64_t segs = (n + stretched - 1) / stretched;
+      const int64_t groups = bh * segs;
+      const double fill = (double)groups / (double)(kMinGroups * ((groups + kMinGroups - 1) / kMinGroups));
+      const double blocks = (double)stretched / kSegQuantum;
+      // (a workgroup spends about two blocks' time on its start-up and the state it loads)
+      const double score = fill * (double)n / (double)(segs * stretched) * blocks / (blocks + 2.0);
+      if (score > best + 0.02) {
+        best = score;
+        best_len = (int)stretched;
+      }
+    }
+    if (best_len) seg_len = best_len;
   }
   const int64_t n_seg_final = (n + seg_len - 1) / seg_len;
   g->b = b;
@@ -196,7 +241,11 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   // a sweep takes the state that enters its first piece.  A pure function of the shape and seg_len, so that a
   // backward call given the forward's seg_len finds the states where the forward left them.
   g->pre_len = seg_len;
-  if (mfma_eligible(d, e, dtype) && !g->combine && !g->fused) {
+  // Only while the chip is not full, though: with more pre-pass workgroups than CUs the long walks overlap with
+  // other workgroups, and whole segments measured 1-3 % faster in all (b*h = 28, n = 65536, 18 segments of 3648
+  // tokens: 1440 us forward + backward against 1484 with halves; b*h = 48, 16 of 4096: 2377 against 2423; at
+  // b*h = 16 and 24, 256 and 240 workgroups, the halves win: 838 against 856, 653 against 663).
+  if (mfma_eligible(d, e, dtype) && !g->combine && !g->fused && (int64_t)b * h * n_seg_final <= kMinGroups) {
     int pre = seg_len;
     while (pre > kPreMaxSeg && pre % (2 * kSegQuantum) == 0) pre /= 2;
     if (pre <= kPreMaxSeg) g->pre_len = pre;

@@ -53,9 +53,12 @@ def test_plan_defaults_and_overrides(lib):
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 4096) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 2048) == (2048, 32, 16 * 32 * 128 * 128 * 4)
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16, 8192) == (8192, 8, 16 * 32 * 128 * 128 * 4)
-    # ragged lengths and narrow rows are planned like the full-width shapes (15 segments of 4608 tokens would
-    # leave CUs idle, so the ragged length keeps 29)
-    assert _abi.plan(1, 16, 65536 + 8, 128, 128, torch.bfloat16)[:2] == (2304, 29)
+    # ragged lengths and narrow rows are planned like the full-width shapes: 8 tokens more than 16 x 4096 still
+    # make 16 segments (of 4224 tokens, pre-pass on halves of them), not 29 shorter ones in two rounds
+    assert _abi.plan(1, 16, 65536 + 8, 128, 128, torch.bfloat16) == (4224, 16, 16 * 32 * 128 * 128 * 4)
+    # where b*h does not divide the chip the segments are stretched until the forward sweep fits one round of 256
+    assert _abi.plan(2, 12, 16384, 128, 128, torch.bfloat16)[:2] == (1664, 10)
+    assert _abi.plan(1, 24, 32768, 128, 128, torch.bfloat16) == (3328, 10, 24 * 20 * 128 * 128 * 4)
     assert _abi.plan(1, 16, 65536, 128, 64, torch.bfloat16) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     # short chunk: 256 tokens per segment at least ...
     assert _abi.plan(1, 16, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
