@@ -59,6 +59,10 @@ def test_plan_defaults_and_overrides(lib):
     # where b*h does not divide the chip the segments are stretched until the forward sweep fits one round of 256
     assert _abi.plan(2, 12, 16384, 128, 128, torch.bfloat16)[:2] == (1664, 10)
     assert _abi.plan(1, 24, 32768, 128, 128, torch.bfloat16) == (3328, 10, 24 * 20 * 128 * 128 * 4)
+    assert _abi.plan(2, 12, 4096, 128, 128, torch.bfloat16)[:2] == (448, 10)      # shorter chunks alike
+    # several rounds where one would need segments beyond ~4096 tokens; the pre-pass then takes whole segments
+    assert _abi.plan(1, 48, 65536, 128, 128, torch.bfloat16) == (4096, 16, 48 * 16 * 128 * 128 * 4)
+    assert _abi.plan(1, 28, 65536, 128, 128, torch.bfloat16)[:2] == (3648, 18)
     assert _abi.plan(1, 16, 65536, 128, 64, torch.bfloat16) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     # short chunk: 256 tokens per segment at least ...
     assert _abi.plan(1, 16, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
