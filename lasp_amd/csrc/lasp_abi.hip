@@ -171,12 +171,12 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     return LASP_E_SEGMENT;
   }
   const bool sweeps16 = mfma_eligible(d, e, dtype) && !fused_eligible(n, d, e, dtype, seg_len_arg, seg_len, n_seg);
-  if (sweeps16 && seg_len_arg == 0 && n_seg > kCombineMaxSeg) {
+  if (sweeps16 && seg_len_arg == 0) {
     // The 16-bit sweeps hold a CU each, so the default plan aims at one round of 256 workgroups in the
     // forward sweep rather than two per CU: longer segments mean fewer states to load and carry (b*h = 16,
     // n = 65536: 4096-token segments, sweeps 193 + 496 us against 201 + 513 with 2048; b*h = 32, n = 16384:
     // 2048 against 1024, 97 + 248 against 102 + 256).
-    while ((int64_t)b * h * ((n + 2 * seg_len - 1) / (2 * seg_len)) >= kMinGroups &&
+    while (n_seg > kCombineMaxSeg && (int64_t)b * h * ((n + 2 * seg_len - 1) / (2 * seg_len)) >= kMinGroups &&
            (n + 2 * seg_len - 1) / (2 * seg_len) > kCombineMaxSeg)
       seg_len *= 2;
     // That leaves between one and two rounds of workgroups, and a round that is only part full costs a whole
@@ -196,7 +196,13 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     const bool over_one_round = bh * ((n + seg_len - 1) / seg_len) > kMinGroups;
     for (int r = 1; r <= 16 && over_one_round; ++r) {
       const int64_t fit = kMinGroups * r / bh;  // segments per (b, h) in r rounds
-      if (fit <= kCombineMaxSeg) continue;
+      // With many (b, h) pairs one round means 2 to 4 segments, which full-width heads sweep without a scan
+      // launch; taken while the segments stay within 1024 tokens, i.e. while the pre-pass's walks stay short
+      // (b*h = 56, n = 2048: 4 segments of 512 tokens, 114 us forward + backward against 151 for 8 of 256;
+      // b*h = 64, n = 3072: 4 of 768, 161 against 200; b*h = 60, n = 4096: 4 of 1024, 203 against 234; but
+      // b*h = 52, n = 8192: 4 of 2048, 384 against 363 for 8 of 1024).
+      const bool few = fit <= kCombineMaxSeg;
+      if (few && (fit < 2 || r > 1 || d != kMaxFeature || e != kMaxFeature)) continue;
       const int64_t len = (n + fit - 1) / fit;
       int64_t stretched = 0;
       if (r > 1) {  // (more than one round: the pre-pass takes whole segments, see pre_len below)
@@ -212,7 +218,7 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
       // forward + backward against 138 for 16 of 256; n = 8192: 10 of 832, 172 against 199; b*h = 40, n = 4096:
       // 6 of 704, 151 against 166); several rounds only pay with long segments
       if (stretched < (r == 1 ? kMinSeg : kPreferredSeg)) break;  // more rounds only make the segments shorter
-      if (stretched > kLongestPlanned) continue;
+      if (stretched > (few ? kPreferredSeg : kLongestPlanned)) continue;
       const int64_t segs = (n + stretched - 1) / stretched;
       const int64_t groups = bh * segs;
       const double fill = (double)groups / (double)(kMinGroups * ((groups + kMinGroups - 1) / kMinGroups));

@@ -60,6 +60,10 @@ def test_plan_defaults_and_overrides(lib):
     assert _abi.plan(2, 12, 16384, 128, 128, torch.bfloat16)[:2] == (1664, 10)
     assert _abi.plan(1, 24, 32768, 128, 128, torch.bfloat16) == (3328, 10, 24 * 20 * 128 * 128 * 4)
     assert _abi.plan(2, 12, 4096, 128, 128, torch.bfloat16)[:2] == (448, 10)      # shorter chunks alike
+    # many heads: one round means 2 to 4 segments, swept without a scan launch while they stay within 1024 tokens
+    assert _abi.plan(1, 64, 2048, 128, 128, torch.bfloat16)[:2] == (512, 4)
+    assert _abi.plan(1, 80, 2048, 128, 128, torch.bfloat16)[:2] == (704, 3)
+    assert _abi.plan(1, 52, 8192, 128, 128, torch.bfloat16)[:2] == (1024, 8)       # 4 x 2048 would not pay
     # several rounds where one would need segments beyond ~4096 tokens; the pre-pass then takes whole segments
     assert _abi.plan(1, 48, 65536, 128, 128, torch.bfloat16) == (4096, 16, 48 * 16 * 128 * 128 * 4)
     assert _abi.plan(1, 28, 65536, 128, 128, torch.bfloat16)[:2] == (3648, 18)
