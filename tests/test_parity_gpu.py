@@ -464,3 +464,47 @@ def test_odd_number_of_pre_pass_pieces(gpu_device):
     got = dict(o=o, dq=kept[0], dk=kept[1], dv=kept[2], kv_out=kv_out, dkv_out=dkv_out)
     for name, t in got.items():
         assert O.rel_err(t.cpu(), ref[name]) <= 2e-2, name
+
+
+@pytest.mark.parametrize("shape", [
+    (1, 28, 40000, 128, 128),   # two rounds of stretched segments, the pre-pass on whole segments
+    (1, 24, 32768 - 8, 128, 128),  # one round of 10 stretched segments cut in two for the pre-pass, ragged
+    (1, 56, 2048, 128, 128),    # many heads: 4 segments swept without a scan
+    (2, 12, 4096, 128, 64),     # one round of short stretched segments, narrow rows
+])
+def test_default_plans_where_heads_do_not_divide_the_chip(gpu_device, shape):
+    """The default plan stretches segments until the forward sweep fills whole rounds of workgroups, which
+    gives segment lengths, piece counts and paths no other test picks: forward + backward with states, the
+    default plan against an explicit seg_len = 1024 (the pre-pass / scan / sweep path on plain segments), states
+    kept against states rebuilt (bit-equal), and -- where the host can afford it -- against the oracle."""
+    from lasp_amd import _abi
+
+    dev = gpu_device
+    b, h, n, d, e = shape
+    g = torch.Generator(device=dev).manual_seed(n + h)
+    mk = lambda *s_: torch.randn(*s_, generator=g, device=dev)
+    q, k = [(mk(b, h, n, d) * d ** -0.5).to(torch.bfloat16) for _ in range(2)]
+    v, do = [mk(b, h, n, e).to(torch.bfloat16) for _ in range(2)]
+    kv, dkv = mk(b, h, d, e) * 0.1, mk(b, h, d, e) * 0.1
+    s = O.slopes_baseline(h).reshape(-1).to(dev)
+    s[::5] = 0.0
+    seg_len, n_seg, _ = _abi.plan(b, h, n, d, e, torch.bfloat16)
+    assert seg_len != 1024 and seg_len % 64 == 0
+    runs = []
+    for seg in (0, 1024):
+        kv_out, dkv_out = torch.empty_like(kv), torch.empty_like(dkv)
+        print(f"b={b} h={h} n={n} d={d} e={e} seg_len={seg} (plan {seg_len} x {n_seg})", flush=True)
+        o, states, sl = _abi.chunk_fwd(q, k, v, s, kv_in=kv, kv_out=kv_out, seg_len=seg)
+        kept = _abi.chunk_bwd(q, k, v, s, do, kv_in=kv, dkv_in=dkv, dkv_out=dkv_out, kv_seg_states=states, seg_len=sl)
+        redone = _abi.chunk_bwd(q, k, v, s, do, kv_in=kv, dkv_in=dkv, dkv_out=None, kv_seg_states=None, seg_len=sl)
+        torch.cuda.synchronize()
+        for a, r in zip(kept, redone):
+            assert torch.equal(a, r)
+        runs.append(dict(o=o, dq=kept[0], dk=kept[1], dv=kept[2], kv_out=kv_out, dkv_out=dkv_out))
+    for name in runs[0]:
+        assert O.rel_err(runs[0][name].cpu(), runs[1][name].float().cpu()) <= 1.2e-2, name
+    if b * h * n <= 200000:
+        c = lambda t: t.cpu()
+        ref = O.ref_chunked(c(q), c(k), c(v), c(s), c(do), c(kv), c(dkv), dtype=torch.float32)
+        for name in runs[0]:
+            assert O.rel_err(runs[0][name].cpu(), ref[name]) <= 2e-2, name
