@@ -184,12 +184,12 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
     // sweep (floor(256 r / (b*h)) segments per (b, h), the segments stretched to cover the chunk) and give
     // segments of 1024 to about 4096 tokens, the one that keeps the most CUs busy -- fill of the last round,
     // times the share of a full segment that the chunk's last segment has, times the share of a workgroup's time
-    // that goes into blocks -- is taken, fewer rounds winning ties.  Measured forward + backward, this plan against the power-of-two one: b*h = 24, n = 16384: 10
-    // segments of 1664 tokens, 334 us against 356; b*h = 24, n = 32768: 647 against 742 (11 segments of 3072 =
-    // 264 workgroups); b*h = 28, n = 65536: 18 of 3648, 1417 against 1493; b*h = 48, n = 65536: 16 of 4096, 2407
-    // against 2715; b*h = 100, n = 8192: 5 of 1664, 669 against 733.  In a one-round plan lengths beyond 2048
-    // tokens stay a multiple of 64 * 2^k with seg_len / 2^k <= kPreMaxSeg, so that the pre-pass can work on equal
-    // pieces of that length.
+    // that goes into blocks -- is taken, fewer rounds winning ties.  Measured forward + backward, this plan
+    // against the power-of-two one: b*h = 24, n = 16384: 10 segments of 1664 tokens, 334 us against 356;
+    // b*h = 24, n = 32768: 647 against 742 (11 segments of 3072 = 264 workgroups); b*h = 28, n = 65536: 18 of
+    // 3648, 1444 against 1493; b*h = 48, n = 65536: 16 of 4096, 2386 against 2715; b*h = 100, n = 8192: 5 of
+    // 1664, 663 against 733.  In a one-round plan lengths beyond 2048 tokens stay a multiple of 64 * 2^k with
+    // seg_len / 2^k <= kPreMaxSeg, so that the pre-pass can work on equal pieces of that length.
     const int64_t bh = (int64_t)b * h;
     double best = 0.0;
     int best_len = 0;
@@ -247,9 +247,10 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
   g->bypass = (mfma_eligible(d, e, dtype) && !g->fused && !g->combine && n_seg_final >= 2) ? 1 : 0;
   // The pre-pass walks a segment serially, and its slow-decay heads walk all of it: beyond 2048 tokens that
   // walk outlasts everything else in the launch (b*h = 16, n = 65536: 71 us at 4096 tokens against 51 at
-  // 2048; at 1024 the extra states cost more again, 62 us and a longer scan).  Long sweep segments are therefore cut in halves (quarters, ...) for the pre-pass and the scan, and
-  // a sweep takes the state that enters its first piece.  A pure function of the shape and seg_len, so that a
-  // backward call given the forward's seg_len finds the states where the forward left them.
+  // 2048; at 1024 the extra states cost more again, 62 us and a longer scan).  Long sweep segments are
+  // therefore cut in halves (quarters, ...) for the pre-pass and the scan, and a sweep takes the state that
+  // enters its first piece.  A pure function of the shape and seg_len, so that a backward call given the
+  // forward's seg_len finds the states where the forward left them.
   g->pre_len = seg_len;
   // Only while the chip is not full, though: with more pre-pass workgroups than CUs the long walks overlap with
   // other workgroups, and whole segments measured 1-3 % faster in all (b*h = 28, n = 65536, 18 segments of 3648
