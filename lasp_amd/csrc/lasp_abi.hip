@@ -144,8 +144,8 @@ constexpr int kFusedMaxWalk = 16;  // blocks
 // (each workgroup re-runs the scan's recurrence over at most kCombineMaxSeg - 1 states of 64 KiB)
 // and the scan launch is dropped; with one segment the pre-pass goes too.  Measured at b*h = 24,
 // n = 2048: 4 segments 84 against 88 us forward + backward, 8 segments 137 against 100 us (the
-// gathers grow with the square of the segment count), hence the limit.  The wave-specialised sweeps gather only as
-// far back as a head's decay reaches and while their other waves fetch the first block; at 7 segments that still
+// gathers grow with the square of the segment count), hence the limit.  The sweeps gather only as far back as a
+// head's decay reaches, and while their feed waves fetch the first block; at 7 segments that still
 // costs what the scan launch saves (b*h = 24, n = 2048: 67 against 69 us per chunk in kernels, 691 against 677 us
 // for the 8-chunk chain replayed from a graph), so the limit stays.
 constexpr int64_t kCombineMaxSeg = 4;

@@ -46,7 +46,7 @@ def test_library_exports_every_declared_symbol(lib):
 def test_plan_defaults_and_overrides(lib):
     from lasp_amd import _abi
 
-    # headline shape: 16 (b,h) pairs -> 16 sweep segments of 4096 tokens = 256 workgroups of the wave-specialised
+    # headline shape: 16 (b,h) pairs -> 16 sweep segments of 4096 tokens = 256 workgroups of the
     # sweeps, one per CU; the pre-pass and the scan work on halves of them, so the workspace holds 32 states per (b,h)
     assert _abi.plan(1, 16, 65536, 128, 128, torch.bfloat16) == (4096, 16, 16 * 32 * 128 * 128 * 4)
     # an explicit seg_len gets the same treatment (the backward is handed the forward's seg_len)

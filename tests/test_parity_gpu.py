@@ -332,9 +332,8 @@ def test_seeded_random_shapes(gpu_device):
         check(got, oracle(inp, s), 1e-4 if dtype == torch.float32 else 2e-2, what=what)
 
 
-def test_seeded_random_shapes_on_the_wave_specialised_kernels(gpu_device):
-    """40 shapes drawn from a fixed seed among those the wave-specialised sweeps serve (16-bit, d = e = 128,
-    whole blocks): 1 to 80 blocks, planned and forced segment lengths from one block upwards -- single-launch,
+def test_seeded_random_shapes_of_whole_blocks(gpu_device):
+    """40 shapes drawn from a fixed seed among the full-width 16-bit shapes of whole blocks (d = e = 128): 1 to 80 blocks, planned and forced segment lengths from one block upwards -- single-launch,
     scan-less (up to 4 segments) and scan paths, sweep segments longer than the pre-pass's 2048-token pieces,
     one-block segments, a short last segment -- with and without incoming states, states kept or recomputed."""
     import random
@@ -364,7 +363,7 @@ def test_seeded_random_shapes_on_the_wave_specialised_kernels(gpu_device):
     (2, 4, 640, 128, 128),     # three segments, the last one short
     (1, 3, 768, 128, 128),     # three segments
     (1, 2, 64, 128, 128), (1, 1, 192, 128, 128),
-    (2, 12, 1024, 128, 128),   # wave-specialised form: six segments of 192 tokens, walks of up to 15 blocks
+    (2, 12, 1024, 128, 128),   # six segments of 192 tokens, walks of up to 15 blocks
     (4, 32, 2048, 128, 128),   # two segments of 1024 tokens, a walk of 16 blocks; 3 * 128 * 2 workgroups backwards
     (2, 3, 700, 128, 128), (1, 4, 513, 128, 128), (1, 2, 333, 128, 128), (1, 2, 1, 128, 128),   # ragged lengths
     (2, 12, 512, 128, 64), (1, 3, 700, 64, 96), (2, 2, 321, 48, 16),                              # narrow rows
