@@ -263,3 +263,31 @@ def test_bench_reads_its_traffic_figures_from_the_committed_profile():
     assert prof["kernels"]["la_bwd3"] >= bench.BYTES_BWD_PER_TH * th
     assert prof["kernels"]["la_apply"] >= bench.BYTES_FWD_PER_TH * th
     assert prof["kernels"]["la_bwd3"] < 2 * bench.BYTES_BWD_PER_TH * th
+
+
+def test_plan_invariants_on_random_shapes(lib):
+    """The plan is what forward and backward agree on: for any shape the default plan must be reproduced by
+    asking for its seg_len explicitly (the binding hands the planned seg_len to both calls), segments are
+    whole blocks that cover the chunk, and the workspace holds a whole number of states, at least one per
+    segment."""
+    import random
+
+    from lasp_amd import _abi
+
+    rng = random.Random(7)
+    for _ in range(3000):
+        b = rng.choice([1, 1, 2, 3, 4, 8])
+        h = rng.choice([1, 2, 3, 7, 8, 12, 16, 20, 24, 28, 32, 40, 48, 52, 64, 96, 100, 128, 200])
+        n = rng.choice([1, 63, 64, 65, 500, 512, 1000, 2048, 2049, 4096, 5000, 8192, 16384, 20000, 32768, 65536,
+                        65544, 100000, 1 << 20]) + rng.choice([0, 0, 0, -8, 8, 72])
+        n = max(n, 1)
+        dtype = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        d, e = rng.choice([(128, 128), (128, 128), (128, 64), (64, 128), (96, 40), (64, 64)])
+        seg_len, n_seg, state_bytes = _abi.plan(b, h, n, d, e, dtype)
+        assert seg_len > 0 and seg_len % 64 == 0 and n_seg == -(-n // seg_len), (b, h, n, d, e, dtype, seg_len, n_seg)
+        padded = (dtype != torch.float32 and d % 8 == 0 and e % 8 == 0) or (dtype == torch.float32 and d == e == 128)
+        one = (128 * 128 if padded else d * e) * 4
+        states, rest = divmod(state_bytes, b * h * one)
+        assert rest == 0 and n_seg <= states <= 64 * n_seg, (b, h, n, d, e, dtype, seg_len, n_seg, state_bytes)
+        if _abi.kernel_path(b, h, n, d, e, dtype) != _abi.PATH_MFMA_FUSED:
+            assert _abi.plan(b, h, n, d, e, dtype, seg_len) == (seg_len, n_seg, state_bytes), (b, h, n, d, e, dtype)
