@@ -797,28 +797,62 @@ la_bwd3(const elem16_t *__restrict__ Q, const elem16_t *__restrict__ K, const el
 //
 // That leaves the workgroups unevenly loaded -- those of slow-decaying heads still read whole
 // segments -- so one workgroup has to be able to pull more than an even share of the memory
-// bandwidth.  512 threads (8 waves, one workgroup per CU): threads 0-255 fetch the Y tile, 256-511
-// the Z tile, each keeping STATE_DEPTH blocks in flight in registers (16 registers per block) on
-// top of the two LDS buffers; wave (wc, rh) owns rows [64 rh, 64 rh + 64) x columns
-// [32 wc, 32 wc + 32) of the state as two accumulator tiles.
+// bandwidth.  512 threads (8 waves): threads 0-255 fetch the Y tile, 256-511 the Z tile, each
+// keeping D blocks in flight in registers (16 registers per block) on top of the two LDS
+// buffers; wave (wc, rh) owns rows [64 rh, 64 rh + 64) x columns [32 wc, 32 wc + 32) of the state
+// as two accumulator tiles.
+//
+// Both tiles stay token-major in LDS, as they are in memory (16-byte copies, Y scaled by the decay
+// weights on the way); the products contract over tokens, so the MFMA operands are fetched with
+// the transposing LDS read.
 constexpr int STATE_THREADS = 512;
-constexpr int STATE_DEPTH = 2;  // blocks in flight per thread in registers (even); deeper measured slower:
-                                // the repeated loads at the end of a walk cost more than the depth gains
+constexpr int LDR = 320;  // bytes per token row (256 + 64: the four rows that one transposing read
+                          // touches per half-wave fall on disjoint banks)
+constexpr int STATE_TILE = BLK * LDR;
+constexpr int STATE_LDS = 2 * 2 * STATE_TILE;  // double-buffered {Y scaled, Z}: 80 KiB, two workgroups fit a CU
+// Blocks in flight per thread in registers (even).  Long walks gain from the deeper pipeline (b*h = 16,
+// n = 65536, 2048-token pieces: 46 us per launch against 49); on short ones the longer start-up costs more
+// than it gains (512-token segments: 13.1 us against 12.5).
+constexpr int STATE_DEPTH_LONG = 4, STATE_DEPTH_SHORT = 2;
+constexpr int STATE_LONG_WALK = 1024;  // tokens per segment from which the deeper pipeline is used
 
-template <class E, bool REV, int MODE>
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4i16 *lds_v4i16;
+// The transposing 8-byte read works in groups of 16 lanes: lane i of a group receives, as element j,
+// element (i % 4) of what lane (4 j + i / 4) of the group addressed.  With lane s of a group addressing
+// token T + s / 4, features f + 4 (s % 4) .. + 3, lane i ends up with feature f + i of tokens T .. T + 3.
+__device__ __forceinline__ u32x2 lds_tr8(const char *p) {
+  const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4i16)(p));
+  return __builtin_bit_cast(u32x2, r);
+}
+// MFMA operand of lane (c, hh): feature f0 + c, tokens t0 + 8 hh .. + 7 (`lane_part` holds the lane's share
+// of the address, see la_seg_state)
+__device__ __forceinline__ u32x4 token_fragment(const char *tile, int lane_part, int f0, int t0) {
+  const char *p = tile + lane_part + t0 * LDR + f0 * 2;
+  const u32x2 lo = lds_tr8(p), hi = lds_tr8(p + 4 * LDR);
+  u32x4 r;
+  r.x = lo.x;
+  r.y = lo.y;
+  r.z = hi.x;
+  r.w = hi.y;
+  return r;
+}
+
+template <class E, bool REV, int MODE, int D>
 __global__ void __launch_bounds__(STATE_THREADS, 1)
 la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, const float *__restrict__ S,
              float *__restrict__ states, Geom g, int skip_seg) {
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
-  constexpr int D = STATE_DEPTH;
-  __shared__ __align__(16) char smem[2][2 * F * LDT];  // double-buffered {Y^T scaled, Z^T}
+  extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, uniform: keeps it in an SGPR
   const int wc = w8 & 3, rh = w8 >> 2;                      // column block and row half of this wave's tiles
   const bool zgrp = w8 >= 4;                                // this wave fetches Z (else Y)
   const int c = lane & 31, hh = lane >> 5;
-  const LoaderRole yr = yz_role(tid & 255);
+  // loader: 16 consecutive threads copy one row, the thread's 16 bytes are features 8 cq .. + 7 of rows
+  // rq, rq + 16, rq + 32, rq + 48
+  const int cq = tid & 15, rq = (tid & 255) >> 4;
 
   // slow-decaying heads (the later ones in the usual slope schedules) have the most to read: first
   const int n_items = g.b * g.h * g.n_seg;
@@ -829,13 +863,13 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   const int yw = NARROW ? g.d : F, zw = NARROW ? g.e : F;  // row widths in elements
   const int tw = zgrp ? zw : yw;                           // of the tile this thread fetches
   const char *Tg = reinterpret_cast<const char *>(zgrp ? Z + row0 * zw : Y + row0 * yw);
-  const int tu = tw / 4;  // 8-byte units per row
+  const int row_bytes = tw * 2;
 
   const float blockdec = decay(sl, (float)BLK);
   float kdec[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int b = 4 * yr.rowq + r;
+    const int b = rq + 16 * r;
     kdec[r] = decay(sl, REV ? (float)b : (float)(BLK - b));
   }
 
@@ -868,50 +902,60 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   // A partial block (the end of a ragged chunk) reads its missing rows as zeros; going
   // forwards it is the last block, and its tokens sit `len - b` (not 64 - b) before the
   // segment end.
-  const uint32_t t_off = lane_offset(yr, 4 * yr.rowq, tu);
-  const PieceMask t_ok = piece_mask(yr, tu);
-  // every address is a workgroup-uniform row pointer plus one per-thread 32-bit offset
+  const uint32_t t_off = (uint32_t)(rq * row_bytes + cq * 16);
+  const bool col_ok = !NARROW || cq * 8 < tw;  // chunks past the row width read as zeros
+  // every address is a workgroup-uniform block pointer plus one per-thread 32-bit offset
   auto issue_loads = [&](u32x4 (&nt)[4], int blk) __attribute__((always_inline)) {
+    typedef const __attribute__((address_space(1))) u32x4 *gmem_u32x4;
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    const gmem_ptr tblk = uniform_ptr(Tg + (int64_t)blk * BLK * tu * 8);
-    const PieceMask all = {true, true};
+    const gmem_ptr tblk = uniform_ptr(Tg + (int64_t)blk * BLK * row_bytes);
+    const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const bool row_ok = !RAGGED || 4 * yr.rowq + r < len;
-      nt[r] = load_row_pieces(tblk, r * tu * 8, t_off, NARROW ? t_ok : all, row_ok);
+      const bool ok = col_ok && (!RAGGED || rq + 16 * r < len);
+      nt[r] = ok ? *reinterpret_cast<gmem_u32x4>(tblk + 16 * r * row_bytes + t_off) : zero;
     }
   };
+  auto scaled = [&](const u32x4 &q, float w) __attribute__((always_inline)) {
+    u32x4 o;
+    o.x = E::pack(elem_f32<E>(q, 0) * w, elem_f32<E>(q, 1) * w);
+    o.y = E::pack(elem_f32<E>(q, 2) * w, elem_f32<E>(q, 3) * w);
+    o.z = E::pack(elem_f32<E>(q, 4) * w, elem_f32<E>(q, 5) * w);
+    o.w = E::pack(elem_f32<E>(q, 6) * w, elem_f32<E>(q, 7) * w);
+    return o;
+  };
+  char *const my_rows = smem + (zgrp ? STATE_TILE : 0) + rq * LDR + cq * 16;
   auto fill_lds = [&](int buf, const u32x4 (&nt)[4], int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
-    if (zgrp) {
-      store_transposed<E, false>(smem[buf] + F * LDT, nt, yr, kdec);
-    } else if (RAGGED && !REV && len != BLK) {
-      float kd[4];
+    char *dst = my_rows + buf * (2 * STATE_TILE);
+    const bool partial = RAGGED && !REV && len != BLK;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) kd[r] = decay(sl, (float)max(len - (4 * yr.rowq + r), 0));
-      store_transposed<E, true>(smem[buf], nt, yr, kd);
-    } else {
-      store_transposed<E, true>(smem[buf], nt, yr, kdec);
+    for (int r = 0; r < 4; ++r) {
+      u32x4 v = nt[r];
+      if (!zgrp) v = scaled(v, partial ? decay(sl, (float)max(len - (rq + 16 * r), 0)) : kdec[r]);
+      *reinterpret_cast<u32x4 *>(dst + 16 * r * LDR) = v;
     }
   };
   // M_NARROW: columns past the width of Z stay zero, as do rows past Y's
   const bool wave_active = !NARROW || (32 * wc < g.e && (rh == 0 || g.d > 64));
+  // the lane's share of a fragment address: token 8 hh + (lane % 16) / 4, feature 16 ((lane / 16) % 2) + 4 (lane % 4)
+  const int lane_part = (8 * hh + ((lane & 15) >> 2)) * LDR + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   auto accumulate = [&](int buf, int blk) __attribute__((always_inline)) {
     const int len = RAGGED && blk == sw.nblk - 1 ? sw.tail : BLK;
     const float bd = RAGGED && len != BLK ? decay(sl, (float)len) : blockdec;
-    const char *yt = smem[buf];
-    const char *zt = yt + F * LDT;
+    const char *yt = smem + buf * (2 * STATE_TILE);
+    const char *zt = yt + STATE_TILE;
     if (wave_active) {
       u32x4 zf[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) zf[u] = lds16(zt + tr_off(32 * wc + c, 2 * u + hh));
+      for (int u = 0; u < 4; ++u) zf[u] = token_fragment(zt, lane_part, 32 * wc, 16 * u);
 #pragma unroll
       for (int T = 0; T < 2; ++T) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[T][r] *= bd;
 #pragma unroll
         for (int u = 0; u < 4; ++u)
-          st[T] = E::mfma(lds16(yt + tr_off(64 * rh + 32 * T + c, 2 * u + hh)), zf[u], st[T]);
+          st[T] = E::mfma(token_fragment(yt, lane_part, 64 * rh + 32 * T, 16 * u), zf[u], st[T]);
       }
     }
   };
@@ -929,17 +973,25 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   fill_lds(0, set[0], block_of(0));
   issue_loads(set[0], block_of(D));
   __syncthreads();
-  for (int i = 0; i < cnt; i += D) {
+  // The walk leaves the loop from the middle of the unrolled body.  Were the exit test left to the loop
+  // head, the compiler would have to assume that any of the D positions can precede the first one, could
+  // no longer tell which register set holds the oldest loads there, and would wait for all of them.
+  for (int i = 0;; i += D) {
+    bool last = false;
 #pragma unroll
     for (int k = 0; k < D; ++k) {  // D is even: LDS buffer (i + k) & 1 == k & 1
-      if (i + k >= cnt) break;
       accumulate(k & 1, block_of(i + k));
       __builtin_amdgcn_sched_barrier(0);
       fill_lds((k + 1) & 1, set[(k + 1) % D], block_of(i + k + 1));
       __builtin_amdgcn_sched_barrier(0);
       issue_loads(set[(k + 1) % D], block_of(i + k + 1 + D));
       __syncthreads();
+      if (i + k + 1 >= cnt) {
+        last = true;
+        break;
+      }
     }
+    if (last) break;
   }
 
   {
@@ -979,15 +1031,25 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
   return (int)hipGetLastError();
 }
 
+template <class E, bool REV, int MODE, int D>
+int launch_state_depth(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
+                       hipStream_t st) {
+  int rc = grant_lds<la_seg_state<E, REV, MODE, D>>(STATE_LDS);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
+  ProfScope prof(KC_STATE, st);
+  la_seg_state<E, REV, MODE, D><<<grid, STATE_THREADS, STATE_LDS, st>>>((const elem16_t *)y, (const elem16_t *)z, s,
+                                                                        states, g, skip_seg);
+  return (int)hipGetLastError();
+}
+
 // skip_seg: the segment whose own state nothing reads (-1: none); its workgroups leave at once
 template <class E, bool REV, int MODE>
 int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
                           hipStream_t st) {
-  const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
-  ProfScope prof(KC_STATE, st);
-  la_seg_state<E, REV, MODE><<<grid, STATE_THREADS, 0, st>>>((const elem16_t *)y, (const elem16_t *)z, s, states, g,
-                                                               skip_seg);
-  return (int)hipGetLastError();
+  return g.seg_len >= STATE_LONG_WALK
+             ? launch_state_depth<E, REV, MODE, STATE_DEPTH_LONG>(y, z, s, states, g, skip_seg, st)
+             : launch_state_depth<E, REV, MODE, STATE_DEPTH_SHORT>(y, z, s, states, g, skip_seg, st);
 }
 
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
