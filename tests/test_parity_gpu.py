@@ -249,7 +249,8 @@ def test_ragged_bf16_length(gpu_device, n, d, e):
         check(got, ref, 2e-2, what=f"ragged n={n} d={d} e={e} cache={cache}")
 
 
-@pytest.mark.parametrize("b,h,n,seg,state", [(1, 2, 256, 64, True), (2, 3, 1024, 256, True), (1, 4, 512, 0, False)])
+@pytest.mark.parametrize("b,h,n,seg,state", [(1, 2, 256, 64, True), (2, 3, 1024, 256, True), (1, 4, 512, 0, False),
+                                             (1, 2, 4096, 2048, True)])  # the last: the pre-pass's deep pipeline
 def test_mfma_fp16(gpu_device, b, h, n, seg, state):
     from lasp_amd import _abi
 
@@ -264,6 +265,10 @@ def test_fp16_narrow_and_ragged(gpu_device):
     inp = make_inputs(1, 3, 333, 64, 96, torch.float16, seed=17, state=True, state_std=1.0)
     s = O.slopes_alibi(3)
     check(run_abi(inp, s, gpu_device), oracle(inp, s), 2e-2, what="fp16 ragged narrow")
+    # segments long enough for the pre-pass's deep pipeline, the last one partial
+    inp = make_inputs(1, 2, 2100, 64, 96, torch.float16, seed=18, state=True, state_std=1.0)
+    s = O.slopes_baseline(2)
+    check(run_abi(inp, s, gpu_device, seg_len=1024), oracle(inp, s), 2e-2, what="fp16 ragged narrow, seg_len=1024")
 
 
 # ---------------------------------------------------------------- fp32 MFMA kernels (d = e = 128)
