@@ -842,7 +842,7 @@ __device__ __forceinline__ u32x4 token_fragment(const char *tile, int lane_part,
 template <class E, bool REV, int MODE, int D>
 __global__ void __launch_bounds__(STATE_THREADS, 1)
 la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, const float *__restrict__ S,
-             float *__restrict__ states, Geom g, int skip_seg) {
+             float *__restrict__ states, Geom g, int skip_seg, int sub) {
   constexpr bool RAGGED = MODE != M_ALIGNED, NARROW = MODE == M_NARROW;
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
@@ -859,7 +859,19 @@ la_seg_state(const elem16_t *__restrict__ Y, const elem16_t *__restrict__ Z, con
   const int n_items = g.b * g.h * g.n_seg;
   const SegWork sw = seg_work(g, n_items - 1 - (int)blockIdx.x);
   if (sw.seg == skip_seg) return;  // the scan's final segment feeds only the outgoing carry
-  const float sl = S[sw.bh % g.h] * LOG2E;
+  const float slope = S[sw.bh % g.h];
+  // Where sweep segments span `sub` > 1 of these segments, a head that takes no part in the scan
+  // (state_dies_in_segment) has readers for one state in `sub` only: a sweep reads the own state of the piece
+  // next to its segment -- the last piece of the segment before it, or going backwards the first piece of the
+  // segment after it -- and the outgoing state, if one is wanted (skip_seg < 0), is formed from the two pieces
+  // visited last.  The other pieces are left out, and their slots in `states` unwritten.
+  if (sub > 1 && state_dies_in_segment(slope, g)) {
+    const int p = sw.seg;
+    bool read = REV ? (p % sub == 0 && p >= sub) : (p % sub == sub - 1 && p + 1 < g.n_seg);
+    if (skip_seg < 0) read = read || (REV ? p <= 1 : p >= g.n_seg - 2);
+    if (!read) return;
+  }
+  const float sl = slope * LOG2E;
   const int64_t row0 = (int64_t)sw.bh * g.n + sw.tok0;
   const int yw = NARROW ? g.d : F, zw = NARROW ? g.e : F;  // row widths in elements
   const int tw = zgrp ? zw : yw;                           // of the tile this thread fetches
@@ -1034,31 +1046,32 @@ int launch_bwd3(const BwdArgs &a, const float *kv_states, const float *dkv_state
 
 template <class E, bool REV, int MODE, int D>
 int launch_state_depth(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
-                       hipStream_t st) {
+                       int sub, hipStream_t st) {
   int rc = grant_lds<la_seg_state<E, REV, MODE, D>>(STATE_LDS);
   if (rc) return rc;
   const unsigned grid = (unsigned)((int64_t)g.b * g.h * g.n_seg);
   ProfScope prof(KC_STATE, st);
   la_seg_state<E, REV, MODE, D><<<grid, STATE_THREADS, STATE_LDS, st>>>((const elem16_t *)y, (const elem16_t *)z, s,
-                                                                        states, g, skip_seg);
+                                                                        states, g, skip_seg, sub);
   return (int)hipGetLastError();
 }
 
-// skip_seg: the segment whose own state nothing reads (-1: none); its workgroups leave at once
+// skip_seg: the segment whose own state nothing reads (-1: none); its workgroups leave at once.
+// sub: segments of `g` per sweep segment (1 unless the plan cut the sweep segments finer for the pre-pass).
 template <class E, bool REV, int MODE>
 int launch_state_skipping(const void *y, const void *z, const float *s, float *states, const Geom &g, int skip_seg,
-                          hipStream_t st) {
+                          hipStream_t st, int sub = 1) {
   return g.seg_len >= STATE_LONG_WALK
-             ? launch_state_depth<E, REV, MODE, STATE_DEPTH_LONG>(y, z, s, states, g, skip_seg, st)
-             : launch_state_depth<E, REV, MODE, STATE_DEPTH_SHORT>(y, z, s, states, g, skip_seg, st);
+             ? launch_state_depth<E, REV, MODE, STATE_DEPTH_LONG>(y, z, s, states, g, skip_seg, sub, st)
+             : launch_state_depth<E, REV, MODE, STATE_DEPTH_SHORT>(y, z, s, states, g, skip_seg, sub, st);
 }
 
 // carry_wanted: whether the scan that follows has to produce the outgoing carry; if not, the
 // segment it visits last (whose own state feeds nothing else) is skipped.
 template <class E, bool REV, int MODE>
 int launch_state(const void *y, const void *z, const float *s, float *states, const Geom &g,
-                 bool carry_wanted, hipStream_t st) {
-  return launch_state_skipping<E, REV, MODE>(y, z, s, states, g, carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1), st);
+                 bool carry_wanted, int sub, hipStream_t st) {
+  return launch_state_skipping<E, REV, MODE>(y, z, s, states, g, carry_wanted ? -1 : (REV ? 0 : g.n_seg - 1), st, sub);
 }
 
 template <class E, int MODE>
@@ -1127,8 +1140,9 @@ int fwd_e(const FwdArgs &a, const Geom &g, hipStream_t st) {
   }
   const bool need_states = g.n_seg > 1 || a.kv_in || a.kv_out;
   const Geom gp = pre_pass_geom(g);
+  const int sub = g.seg_len / g.pre_len;  // pre-pass segments per sweep segment
   if (need_states) {
-    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, gp, a.kv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.seg_states, gp, a.kv_out != nullptr, sub, st))) return rc;
     if ((rc = launch_segment_scan(a.seg_states, a.kv_in, a.kv_out, a.s, gp, 0, st))) return rc;
   }
   return launch_apply<E, false, false, SRC_SCANNED, MODE>(a.q, a.k, a.v, a.s, need_states ? a.seg_states : nullptr,
@@ -1150,15 +1164,16 @@ int bwd_e(const BwdArgs &a, const Geom &g, hipStream_t st) {
                                                 g.n_seg > 1 ? a.ws_dkv : nullptr, g, st);
   }
   const Geom gp = pre_pass_geom(g);
+  const int sub = g.seg_len / g.pre_len;  // pre-pass segments per sweep segment
   const float *kv_states = a.kv_seg_states;
   if (!kv_states && (g.n_seg > 1 || a.kv_in)) {
-    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, gp, false, st))) return rc;
+    if ((rc = launch_state<E, false, MODE>(a.k, a.v, a.s, a.ws_kv, gp, false, sub, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_kv, a.kv_in, nullptr, a.s, gp, 0, st))) return rc;
     kv_states = a.ws_kv;
   }
   const float *dkv_states = nullptr;
   if (g.n_seg > 1 || a.dkv_in || a.dkv_out) {
-    if ((rc = launch_state<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, gp, a.dkv_out != nullptr, st))) return rc;
+    if ((rc = launch_state<E, true, MODE>(a.q, a.d_o, a.s, a.ws_dkv, gp, a.dkv_out != nullptr, sub, st))) return rc;
     if ((rc = launch_segment_scan(a.ws_dkv, a.dkv_in, a.dkv_out, a.s, gp, 1, st))) return rc;
     dkv_states = a.ws_dkv;
   }
