@@ -812,7 +812,7 @@ constexpr int STATE_TILE = BLK * LDR;
 constexpr int STATE_LDS = 2 * 2 * STATE_TILE;  // double-buffered {Y scaled, Z}: 80 KiB
 // Blocks in flight per thread in registers (even).  Long walks gain from the deeper pipeline (b*h = 16,
 // n = 65536, 2048-token pieces: 46 us per launch against 49); on short ones the longer start-up costs more
-// than it gains (512-token segments: 13.1 us against 12.5).  The shallow form stays within 128 registers, so two
+// than it gains (320-token segments: 13.1 us against 12.4).  The shallow form stays within 128 registers, so two
 // workgroups share a CU; the deep one runs one per CU (squeezed into 128 registers it spills and measured slower).
 constexpr int STATE_DEPTH_LONG = 4, STATE_DEPTH_SHORT = 2;
 constexpr int STATE_LONG_WALK = 1024;  // tokens per segment from which the deeper pipeline is used
