@@ -470,6 +470,47 @@ def test_odd_number_of_pre_pass_pieces(gpu_device):
         assert O.rel_err(t.cpu(), ref[name]) <= 2e-2, name
 
 
+def test_unwritten_workspace_slots_are_never_read(gpu_device, monkeypatch):
+    """Heads that take no part in the scan get only the piece states that something reads (one per sweep
+    segment, and the two visited last for the outgoing state); the other slots of the workspace stay as they
+    were allocated.  With every fresh allocation of the binding poisoned with NaN (workspaces and outputs alike)
+    the results must be finite and bit-identical to those of a run on zeroed allocations."""
+    from lasp_amd import _abi
+
+    dev = gpu_device
+    b, h, n, d = 1, 4, 4096 * 5 - 2048 - 8, 128
+    inp = make_inputs(b, h, n, d, d, torch.bfloat16, seed=92, scale=d ** -0.5, state=True, device=dev)
+    s = O.slopes_baseline(16).reshape(-1)[[0, 9, 14, 15]].contiguous().to(dev)  # two heads outside the scan, two in it
+    real_empty, real_empty_like = torch.empty, torch.empty_like
+
+    def run(fill, carry):
+        def filled(t):
+            return t.fill_(fill) if t.is_floating_point() else t
+        monkeypatch.setattr(torch, "empty", lambda *a, **k: filled(real_empty(*a, **k)))
+        monkeypatch.setattr(torch, "empty_like", lambda *a, **k: filled(real_empty_like(*a, **k)))
+        try:
+            kv_out = torch.empty_like(inp["kv"]) if carry else None
+            dkv_out = torch.empty_like(inp["dkv"]) if carry else None
+            o, states, sl = _abi.chunk_fwd(inp["q"], inp["k"], inp["v"], s, kv_in=inp["kv"], kv_out=kv_out, seg_len=4096)
+            kept = _abi.chunk_bwd(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=inp["dkv"],
+                                  dkv_out=dkv_out, kv_seg_states=states, seg_len=sl)
+            redone = _abi.chunk_bwd(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=inp["dkv"],
+                                    dkv_out=None, kv_seg_states=None, seg_len=sl)
+            torch.cuda.synchronize()
+        finally:
+            monkeypatch.undo()
+        out = [o, *kept, *redone] + ([kv_out, dkv_out] if carry else [])
+        return out, states
+
+    for carry in (True, False):
+        clean, _ = run(0.0, carry)
+        poisoned, states = run(float("nan"), carry)
+        assert torch.isnan(states).any(), "the plan of this shape leaves pieces out: some slots stay unwritten"
+        for a, r in zip(clean, poisoned):
+            assert torch.isfinite(r.float()).all()
+            assert torch.equal(a, r)
+
+
 @pytest.mark.parametrize("shape", [
     (1, 28, 40000, 128, 128),   # two rounds of stretched segments, the pre-pass on whole segments
     (1, 24, 32768 - 8, 128, 128),  # one round of 10 stretched segments cut in two for the pre-pass, ragged
