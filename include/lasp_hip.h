@@ -15,7 +15,7 @@
  *                    piece of a long segment; each d x e, or zero-extended to 128 x 128): opaque to the caller
  *
  * Alignment: q, k, v, o, do, dq, dk, dv start on a 16-byte boundary (the kernels
- * fetch rows with 8-byte loads and store them with 16-byte stores; rows of d or e
+ * fetch rows with 8- and 16-byte loads and store them with 16-byte stores; rows of d or e
  * 16-bit elements with d, e multiples of 8 keep every row aligned as well); s, the
  * states and the workspaces on a 4-byte boundary.  A pointer that is not returns
  * LASP_E_ALIGN.
@@ -131,7 +131,8 @@ int lasp_inplace_ok(int b, int h, int64_t n, int d, int e, int dtype, int seg_le
  * that overlap without being the same.
  * seg_states: workspace of `state_bytes` (lasp_plan); on return it holds per-segment states (opaque:
  * the state entering each segment; each segment's own contribution with few segments, and for
- * heads whose decay wipes a state within one segment, which the scan leaves out), which
+ * heads whose decay wipes a state within one segment, which the scan leaves out; slots that nothing
+ * reads are left unwritten), which
  * lasp_chunk_bwd accepts as `kv_seg_states` -- for the same inputs, seg_len and kv_in -- to skip
  * recomputing them.  It may be NULL when n_seg == 1 and kv_in == NULL and kv_out == NULL, and on
  * LASP_PATH_MFMA_FUSED.
