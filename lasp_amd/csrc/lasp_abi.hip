@@ -155,11 +155,39 @@ bool fused_eligible(int64_t n, int d, int e, int dtype, int seg_len_arg, int seg
   return (n_seg - 1) * per_seg <= kFusedMaxWalk;
 }
 
+// Default segment length of the fp32 MFMA kernels and the generic kernels, which run two (or more) workgroups
+// per CU and are bound by arithmetic: what counts is that every CU gets the same number of workgroups.  Of the
+// power-of-two lengths that give the forward sweep at least one workgroup per CU, the one with the smallest
+// load per CU -- ceil(workgroups / 256) x (seg_len + 64 tokens for the state each workgroup loads and leaves) --
+// is taken, longer segments (fewer states to scan) winning ties; a single segment of 1024 tokens or more is
+// then cut in two when the chunk has more than one, because two workgroups on a CU fill each other's waits.
+// Measured forward + backward in fp32, d = e = 128, this rule against the one of the 16-bit sweeps:
+// b*h = 24, n = 16384: 512 tokens, 1555 us against 1783 (1024: 384 workgroups, half the CUs with two);
+// b*h = 4, n = 8192: 128 tokens, 181 against 231; b*h = 8, n = 4096: 128, 173 against 228; b*h = 16, n = 1024:
+// 64, 108 against 176; b*h = 1, n = 8192: 64, 109 against 179; b*h = 24, n = 2048: 128, 272 against 280; equal
+// within 3 % on the other shapes tried (b*h = 1 ... 256, n = 1024 ... 262144).
+int two_per_cu_seg_len(int b, int h, int64_t n) {
+  const int64_t bh = (int64_t)b * h;
+  auto groups = [&](int64_t len) { return bh * ((n + len - 1) / len); };
+  int64_t best = kSegQuantum, best_load = -1;
+  for (int64_t len = kSegQuantum; len <= kMaxSeg; len *= 2) {
+    if (groups(len) < kMinGroups && len > kSegQuantum) break;  // (the shortest length stands where nothing fills the chip)
+    const int64_t load = ((groups(len) + kMinGroups - 1) / kMinGroups) * (len + kSegQuantum);
+    if (best_load < 0 || load <= best_load) {
+      best = len;
+      best_load = load;
+    }
+    if (len >= n) break;
+  }
+  if (best >= kPreferredSeg && best < n && groups(best) <= kMinGroups) best /= 2;
+  return (int)best;
+}
+
 int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geom *g) {
   int rc = check_shape(b, h, n, d, e, dtype);
   if (rc) return rc;
   const int seg_len_arg = seg_len;
-  if (seg_len == 0) seg_len = default_seg_len(b, h, n);
+  if (seg_len == 0) seg_len = mfma_eligible(d, e, dtype) ? default_seg_len(b, h, n) : two_per_cu_seg_len(b, h, n);
   if (seg_len < 0 || seg_len % kSegQuantum != 0) {
     set_error("seg_len=%d must be a positive multiple of %d (or 0 for the default)", seg_len,
               kSegQuantum);

@@ -85,6 +85,28 @@ def test_plan_defaults_and_overrides(lib):
     assert ns == 1 and sl >= 4096
 
 
+def test_default_plan_of_the_kernels_that_run_two_workgroups_per_cu(lib):
+    """fp32 and the generic kernels are bound by arithmetic and share a CU: the default plan gives every CU the
+    same number of workgroups (a power-of-two segment length; the expectations are the fastest lengths measured)."""
+    from lasp_amd import _abi
+
+    f32 = lambda b, h, n: _abi.plan(b, h, n, 128, 128, torch.float32)[:2]
+    assert f32(2, 12, 2048) == (128, 16)       # configuration 0: 384 workgroups
+    assert f32(2, 12, 16384) == (512, 32)      # 768 = three per CU; 1024 tokens would leave half the CUs with two
+    assert f32(1, 16, 65536) == (2048, 32)     # 512: a one-per-CU plan of 1024 tokens and more is cut in two
+    assert f32(1, 32, 16384) == (1024, 16)
+    assert f32(1, 4, 8192) == (128, 64)        # exactly one per CU
+    assert f32(1, 1, 65536) == (256, 256)
+    assert f32(1, 1, 8192) == (64, 128)        # never fills the chip: the shortest segments
+    assert f32(1, 16, 1024) == (64, 16)
+    assert f32(8, 32, 1024) == (1024, 1)       # one segment per (b, h) already fills it: no pre-pass, no scan
+    assert f32(1, 1, 100) == (64, 2)
+    # 16-bit shapes that the MFMA kernels do not take (e not a multiple of 8) are planned the same way
+    assert _abi.plan(2, 12, 2048, 128, 60, torch.bfloat16)[:2] == (128, 16)
+    # an explicit seg_len is taken as given
+    assert _abi.plan(2, 12, 2048, 128, 128, torch.float32, 320)[:2] == (320, 7)
+
+
 def test_plan_rejects_bad_arguments(lib):
     from lasp_amd import _abi
 
