@@ -100,8 +100,14 @@ int default_seg_len(int b, int h, int64_t n) {
   // shorter serial walk (b*h = 12, n = 2048: 60 against 67 us forward + backward; b*h = 6, n = 4096:
   // 62 against 71).  Not for one or two (b, h) pairs, where the longer scan costs more than that, and
   // not for chunks short enough for the single-launch kernels, whose choice this must not disturb.
+  // Only where the shorter segments do not cost the backward sweep (one workgroup per CU) another round:
+  // b*h = 4, n = 4096: 22 segments of 192 tokens are 264 workgroups, 56 us against 51 for 16 of 256; b*h = 8,
+  // n = 2048: 52 against 49; b*h = 6, n = 3072: 54 against 52 -- and the other way round wherever the rounds
+  // stay the same (b*h = 3 ... 14, n = 2048 ... 4096: 2-6 us faster on 192).
   constexpr int kShortSeg = 3 * kSegQuantum;
-  if (len == kMinSeg && bh >= 3 && n > 3 * kMinSeg && 3 * bh * ((n + kShortSeg - 1) / kShortSeg) <= kTargetGroups)
+  auto bwd_rounds = [&](int64_t l) { return (3 * bh * ((n + l - 1) / l) + kMinGroups - 1) / kMinGroups; };
+  if (len == kMinSeg && bh >= 3 && n > 3 * kMinSeg && 3 * bh * ((n + kShortSeg - 1) / kShortSeg) <= kTargetGroups &&
+      bwd_rounds(kShortSeg) <= bwd_rounds(kMinSeg))
     len = kShortSeg;
   // The backward sweep runs three workgroups per segment.  When those exceed what the chip holds at
   // once by a little (up to a quarter), the stragglers cost it a second round; segments up to two
@@ -116,6 +122,14 @@ int default_seg_len(int b, int h, int64_t n) {
       if (longer <= len + 2 * kSegQuantum) len = longer;
     }
   }
+  // One or two (b, h) pairs cannot fill the chip with segments of 256 tokens and more; there the sweeps (serial in
+  // the blocks of a segment) are traded against the scan (serial in the segments): about 2 sqrt(n) tokens per
+  // segment.  Forward + backward, b*h = 1: n = 32768, 64 segments of 512 tokens 81 us against 93 for 128 of 256;
+  // n = 65536: 120 for 128 of 512 against 148; n = 131072: 177 for 128 of 1024 against 190 for 256 of 512 and 203
+  // for 64 of 2048; n = 262144: 291 for 256 of 1024 against 307 for 128 of 2048; b*h = 2, n = 32768: 104 against 117.
+  int64_t balanced = kMinSeg;
+  while (balanced * balanced < 4 * n) balanced *= 2;
+  if (balanced > kMinSeg && balanced > len && bh * ((n + balanced - 1) / balanced) <= kMinGroups) len = balanced;
   if (len > kMaxSeg) len = kMaxSeg;
   return (int)len;
 }
@@ -229,8 +243,13 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
       // (b*h = 56, n = 2048: 4 segments of 512 tokens, 114 us forward + backward against 151 for 8 of 256;
       // b*h = 64, n = 3072: 4 of 768, 161 against 200; b*h = 60, n = 4096: 4 of 1024, 203 against 234; but
       // b*h = 52, n = 8192: 4 of 2048, 384 against 363 for 8 of 1024).
+      // Where such a plan fills the chip to 7/8 and more it is taken up to 2048 tokens and over two rounds as well
+      // (b*h = 64, n = 8192: 4 of 2048, 413 us against 438 for 8 of 1024; b*h = 128, n = 4096: 2 of 2048, 408
+      // against 430; b*h = 128, n = 8192: 4 of 2048 in two rounds, 808 against 860 for 6 of 1408 in three; b*h = 120, n = 4096: 2 of 2048, 394 against 411; but b*h = 52, n = 8192,
+      // 208 of 256 CUs: 380 against 360).
       const bool few = fit <= kCombineMaxSeg;
-      if (few && (fit < 2 || r > 1 || d != kMaxFeature || e != kMaxFeature)) continue;
+      const bool few_fills = few && bh * fit * 8 >= kMinGroups * r * 7;
+      if (few && (fit < 2 || r > (few_fills ? 2 : 1) || d != kMaxFeature || e != kMaxFeature)) continue;
       const int64_t len = (n + fit - 1) / fit;
       int64_t stretched = 0;
       if (r > 1) {  // (more than one round: the pre-pass takes whole segments, see pre_len below)
@@ -246,7 +265,7 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
       // forward + backward against 138 for 16 of 256; n = 8192: 10 of 832, 172 against 199; b*h = 40, n = 4096:
       // 6 of 704, 151 against 166); several rounds only pay with long segments
       if (stretched < (r == 1 ? kMinSeg : kPreferredSeg)) break;  // more rounds only make the segments shorter
-      if (stretched > (few ? kPreferredSeg : kLongestPlanned)) continue;
+      if (stretched > (few ? (few_fills ? 2 * kPreferredSeg : kPreferredSeg) : kLongestPlanned)) continue;
       const int64_t segs = (n + stretched - 1) / stretched;
       const int64_t groups = bh * segs;
       const double fill = (double)groups / (double)(kMinGroups * ((groups + kMinGroups - 1) / kMinGroups));
@@ -327,7 +346,8 @@ int check_device(const char *call, const void *q) {
 }
 
 // In-place state update (out == in).  The scan kernel reads the incoming carry and writes the
-// outgoing one from the same thread, so the pre-pass / scan / sweep path takes it.  On the paths
+// outgoing one from the same thread, and for the heads it leaves out it parks the incoming carry in
+// the workspace, where the sweeps take it from; so the pre-pass / scan / sweep path takes it.  On the paths
 // where the sweeps combine the states themselves every workgroup of a (b, h) reads the incoming
 // state when it starts and one of them writes the outgoing state when it ends; nothing orders a
 // late starter against an early finisher, so in place is only safe when one workgroup does both.

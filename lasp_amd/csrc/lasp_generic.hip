@@ -364,8 +364,8 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
   if (state_dies_in_segment(s, g)) {
     // This head's own states stay as the pre-pass wrote them (the sweeps read the neighbour's).  Only the
     // outgoing carry is formed, from the two segments visited last: anything older has faded below 2^-24.
+    const int prev = reverse ? 1 : g.n_seg - 2, end = reverse ? 0 : g.n_seg - 1;
     if (carry_out && in_carry) {
-      const int prev = reverse ? 1 : g.n_seg - 2, end = reverse ? 0 : g.n_seg - 1;
       ScanVec<W> a, b;
       a.load(p + (int64_t)prev * sde);
       b.load(p + (int64_t)end * sde);
@@ -373,6 +373,10 @@ segment_scan_kernel(float *__restrict__ states, const float *carry_in, float *ca
 #pragma unroll
       for (int w = 0; w < W; ++w) carry_out[cidx + w] = fmaf(f, a.v[w], b.v[w]);
     }
+    // The incoming carry (read above, before the outgoing one was written: the two may be the same memory)
+    // moves into the slot of the segment visited last, whose own state nothing reads from here on; the sweep
+    // of the segment visited first takes it from there, zero-extended like every state of the workspace.
+    if (carry_in) run.store(p + (int64_t)end * sde);
     return;
   }
   // The loads do not depend on the recurrence: a batch of segment states is fetched while the

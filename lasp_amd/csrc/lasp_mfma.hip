@@ -556,10 +556,10 @@ ws_body(const elem16_t *__restrict__ X, const elem16_t *__restrict__ Y, const el
         else
           src = states + ((int64_t)sw.bh * g.pre_n + nb) * (F * F);
       }
-      if (!from_carry)
-        add_state(src, 0.f);
-      else if (carry_in != nullptr)
-        add_carry();
+      // (for such a head the scan kernel has parked the chunk's incoming state in the slot of the piece it
+      // visits last, so that nothing reads `carry_in`'s memory once the outgoing state may have replaced it)
+      if (from_carry) src = states + ((int64_t)sw.bh * g.pre_n + (REV ? 0 : g.pre_n - 1)) * (F * F);
+      if (!from_carry || carry_in != nullptr) add_state(src, 0.f);
     }
   } else {
     // `states` holds the segments' OWN states.  The scan's recurrence, St <- l^len_j St + own_j over the

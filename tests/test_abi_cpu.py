@@ -77,6 +77,20 @@ def test_plan_defaults_and_overrides(lib):
     # 8 segments of 256 would give the backward 3 * 24 * 8 = 576 workgroups, a few more than fit at once:
     # 7 segments of 320 (the last one 128) keep it to one round
     assert _abi.plan(2, 12, 2048, 128, 128, torch.bfloat16)[:2] == (320, 7)
+    # ... and only where the shorter segments do not cost the backward sweep's 3 workgroups per segment another round
+    assert _abi.plan(1, 4, 4096, 128, 128, torch.bfloat16)[:2] == (256, 16)   # 22 x 192 would be 264 workgroups
+    assert _abi.plan(1, 8, 2048, 128, 128, torch.bfloat16)[:2] == (256, 8)
+    assert _abi.plan(1, 6, 4096, 128, 128, torch.bfloat16)[:2] == (192, 22)   # two rounds either way
+    # one or two (b, h) pairs and a long chunk: about 2 sqrt(n) tokens per segment (sweeps against scan)
+    assert _abi.plan(1, 1, 32768, 128, 128, torch.bfloat16)[:2] == (512, 64)
+    assert _abi.plan(1, 1, 131072, 128, 128, torch.bfloat16)[:2] == (1024, 128)
+    assert _abi.plan(1, 2, 32768, 128, 128, torch.bfloat16)[:2] == (512, 64)
+    assert _abi.plan(1, 1, 16384, 128, 128, torch.bfloat16)[:2] == (256, 64)
+    # few segments that fill the chip (to 7/8 and more) are taken up to 2048 tokens, and over two rounds
+    assert _abi.plan(1, 64, 8192, 128, 128, torch.bfloat16)[:2] == (2048, 4)
+    assert _abi.plan(1, 128, 4096, 128, 128, torch.bfloat16)[:2] == (2048, 2)
+    assert _abi.plan(1, 128, 8192, 128, 128, torch.bfloat16)[:2] == (2048, 4)
+    assert _abi.plan(1, 52, 8192, 128, 128, torch.bfloat16)[:2] == (1024, 8)   # 208 of 256 CUs: not worth the long walks
     # ragged n: last segment shorter
     assert _abi.plan(1, 1, 300, 64, 32, torch.float32, 64)[:2] == (64, 5)
     assert _abi.plan(1, 1, 300, 64, 32, torch.float32, 64)[2] == 5 * 64 * 32 * 4

@@ -470,6 +470,44 @@ def test_odd_number_of_pre_pass_pieces(gpu_device):
         assert O.rel_err(t.cpu(), ref[name]) <= 2e-2, name
 
 
+@pytest.mark.parametrize("n,seg_len", [(4096, 256), (4096 * 5 - 2048 - 8, 4096)])
+def test_in_place_state_update_with_heads_outside_the_scan(gpu_device, n, seg_len):
+    """kv_out = kv_in (and dkv_out = dkv_in) on the pre-pass / scan / sweep path.  The scan writes the outgoing
+    state before the sweeps run; a head that takes no part in the scan needs the INCOMING state in the sweep of
+    its first segment, which therefore must not come from the caller's buffer any more.  In place and out of
+    place have to agree bit for bit, for heads in the scan and outside it, with the forward's states kept or not."""
+    from lasp_amd import _abi
+
+    dev = gpu_device
+    b, h, d = 1, 4, 128
+    inp = make_inputs(b, h, n, d, d, torch.bfloat16, seed=93, scale=d ** -0.5, state=True, device=dev)
+    s = O.slopes_baseline(16).reshape(-1)[[0, 9, 14, 15]].contiguous().to(dev)
+    assert _abi.inplace_ok(b, h, n, d, d, torch.bfloat16, seg_len, False)
+    assert _abi.inplace_ok(b, h, n, d, d, torch.bfloat16, seg_len, True)
+
+    def run(in_place):
+        kv, dkv = inp["kv"].clone(), inp["dkv"].clone()
+        kv_out = kv if in_place else torch.empty_like(kv)
+        dkv_out = dkv if in_place else torch.empty_like(dkv)
+        o, states, sl = _abi._chunk_fwd_exact(inp["q"], inp["k"], inp["v"], s, kv_in=kv, kv_out=kv_out, seg_len=seg_len)
+        kept = _abi._chunk_bwd_exact(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=dkv,
+                                     dkv_out=dkv_out, kv_seg_states=states, seg_len=sl)
+        dkv2 = inp["dkv"].clone()
+        redone = _abi._chunk_bwd_exact(inp["q"], inp["k"], inp["v"], s, inp["do"], kv_in=inp["kv"], dkv_in=dkv2,
+                                       dkv_out=dkv2 if in_place else torch.empty_like(dkv2), kv_seg_states=None,
+                                       seg_len=sl)
+        torch.cuda.synchronize()
+        return [o, kv_out, *kept, dkv_out, *redone]
+
+    for a, r in zip(run(False), run(True)):
+        assert torch.equal(a, r)
+    cpu = {k_: t.cpu() for k_, t in inp.items()}
+    ref = O.ref_chunked(cpu["q"], cpu["k"], cpu["v"], s.cpu(), cpu["do"], cpu["kv"], cpu["dkv"], dtype=torch.float32)
+    got = run(True)
+    for name, t in zip(("o", "kv_out", "dq", "dk", "dv", "dkv_out"), got):
+        assert O.rel_err(t.cpu(), ref[name]) <= 2e-2, name
+
+
 def test_unwritten_workspace_slots_are_never_read(gpu_device, monkeypatch):
     """Heads that take no part in the scan get only the piece states that something reads (one per sweep
     segment, and the two visited last for the outgoing state); the other slots of the workspace stay as they
