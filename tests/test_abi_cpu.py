@@ -59,7 +59,12 @@ def test_plan_defaults_and_overrides(lib):
     # where b*h does not divide the chip the segments are stretched until the forward sweep fits one round of 256
     assert _abi.plan(2, 12, 16384, 128, 128, torch.bfloat16)[:2] == (1664, 10)
     assert _abi.plan(1, 24, 32768, 128, 128, torch.bfloat16) == (3328, 10, 24 * 20 * 128 * 128 * 4)
-    assert _abi.plan(2, 12, 4096, 128, 128, torch.bfloat16)[:2] == (448, 10)      # shorter chunks alike
+    assert _abi.plan(1, 40, 4096, 128, 128, torch.bfloat16)[:2] == (704, 6)       # shorter chunks alike
+    # ... and where the segments are short, a few longer ones that save the backward sweep (three workgroups per
+    # segment) a round are taken instead: 7 x 3 x 24 = 504 workgroups are two rounds, 10 x 3 x 24 three
+    assert _abi.plan(2, 12, 4096, 128, 128, torch.bfloat16)[:2] == (640, 7)
+    assert _abi.plan(1, 12, 8192, 128, 128, torch.bfloat16)[:2] == (640, 13)
+    assert _abi.plan(2, 12, 8192, 128, 128, torch.bfloat16)[:2] == (832, 10)      # not beyond about 10 blocks
     # many heads: one round means 2 to 4 segments, swept without a scan launch while they stay within 1024 tokens
     assert _abi.plan(1, 64, 2048, 128, 128, torch.bfloat16)[:2] == (512, 4)
     assert _abi.plan(1, 80, 2048, 128, 128, torch.bfloat16)[:2] == (704, 3)
