@@ -278,17 +278,19 @@ int make_geom(int b, int h, int64_t n, int d, int e, int dtype, int seg_len, Geo
       }
     }
     if (best_len) seg_len = best_len;
-    // The backward sweep runs three workgroups per segment.  With short segments in one (nearly full) forward round, a few
+    // The backward sweep runs three workgroups per segment.  With short segments in one forward round that is at least three quarters full, a few
     // longer ones that save the backward a round are worth it: (1 + rounds) x (blocks + 3) is what a chunk costs,
     // 3 blocks standing for a workgroup's start-up and state traffic (b*h = 24, n = 4096: 7 segments of 640
     // tokens, 106 us forward + backward against 112 for 10 of 448; b*h = 12, n = 8192: 13 of 640, 108 against 112).
     // The longer segments win while they stay below about 10 blocks; beyond that the rounds saved cost more in
     // the forward sweep than they bring (b*h = 24, n = 8192: 10 of 832, 168 against 179 for 7 of 1216).
+    // With the forward round less than three quarters full the outcome is mixed (half full: b*h = 2, n = 16384, 70 us
+    // against 78, but b*h = 6, n = 6144, 79 against 67), so those plans stay.
     {
       const int64_t segs = (n + seg_len - 1) / seg_len;
       const int64_t rounds = (3 * bh * segs + kMinGroups - 1) / kMinGroups;
       const int64_t fewer = rounds >= 2 ? kMinGroups * (rounds - 1) / (3 * bh) : 0;  // segments per (b, h)
-      if (bh * segs <= kMinGroups && bh * segs * 8 >= kMinGroups * 7 && fewer > kCombineMaxSeg && fewer < segs) {
+      if (bh * segs <= kMinGroups && bh * segs * 4 >= kMinGroups * 3 && fewer > kCombineMaxSeg && fewer < segs) {
         int64_t longer = (n + fewer - 1) / fewer;
         longer = ((longer + kSegQuantum - 1) / kSegQuantum) * kSegQuantum;
         const int64_t cost_now = (1 + rounds) * (seg_len / kSegQuantum + 3);
