@@ -178,38 +178,12 @@ __device__ __forceinline__ void store_transposed(char *tile, const u32x4 (&rows)
   }
 }
 
-// the thread's two 8-byte pieces of one 128-feature row (pointer to the row start)
-__device__ __forceinline__ u32x4 load_row_pieces(const u32x2 *row, const LoaderRole &role) {
-  const u32x2 lo = row[4 * role.G + role.j];
-  const u32x2 hi = row[4 * role.G + 2 + role.j];
-  u32x4 r;
-  r.x = lo.x;
-  r.y = lo.y;
-  r.z = hi.x;
-  r.w = hi.y;
-  return r;
-}
-
-// Narrow or partial tiles: a thread's two pieces of the row that starts `row_bytes` (uniform
-// across the workgroup) past `tile`, at the thread's own byte offset `lane_off` (32 bits,
+// A thread's two 8-byte pieces of the row that starts `row_bytes` (uniform across the workgroup) past
+// the block pointer `tile` (scalar, see uniform_ptr), at the thread's own byte offset `lane_off` (32 bits,
 // loop-invariant); a piece that lies beyond the row width, or the whole row, reads as zeros.
 struct PieceMask {
   bool lo, hi;
 };
-__device__ __forceinline__ u32x4 load_row_pieces(const char *tile, int64_t row_bytes, uint32_t lane_off,
-                                                 PieceMask ok, bool row_ok) {
-  const char *p = tile + row_bytes;
-  const u32x2 zero = {0u, 0u};
-  const u32x2 lo = (row_ok && ok.lo) ? *reinterpret_cast<const u32x2 *>(p + lane_off) : zero;
-  const u32x2 hi = (row_ok && ok.hi) ? *reinterpret_cast<const u32x2 *>(p + lane_off + 16) : zero;
-  u32x4 r;
-  r.x = lo.x;
-  r.y = lo.y;
-  r.z = hi.x;
-  r.w = hi.y;
-  return r;
-}
-// the same through a scalar block pointer (see uniform_ptr)
 __device__ __forceinline__ u32x4 load_row_pieces(gmem_ptr tile, int row_bytes, uint32_t lane_off, PieceMask ok,
                                                  bool row_ok) {
   typedef const __attribute__((address_space(1))) u32x2 *gmem_u32x2;
